@@ -1,0 +1,132 @@
+/*
+ * sideaware.so for MI355X (gfx950): C ABI.
+ *
+ * A drop-in for the reference library's `extern "C"` surface (sideaware.cu:1278-1524): the
+ * same names, parameter order and widths, so ctypes bindings written for the reference
+ * (test.py:18-39, example_wrapper.py:53-80) and PyTorch's pluggable allocator
+ * (test.py:14, example_wrapper.py:46) bind without change.  Streams are `hipStream_t`
+ * (an opaque pointer, 0 = the default stream); status codes are `hipError_t` values
+ * (0 = success, 2 = out of memory).
+ *
+ * No entry point throws or aborts.  A call that cannot do its work prints one line to stderr,
+ * records it for sideaware_last_error(), and returns (null / nonzero where there is a return
+ * value).
+ *
+ * Where the reference speaks of the two L2 "sides" of an H100 and of SMs, this library speaks
+ * of the XCDs of an MI355X (8, each with a private 4 MiB L2) and of CUs; each query below says
+ * what it returns here.
+ */
+#ifndef SIDEAWARE_H
+#define SIDEAWARE_H
+
+#include <stdbool.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* sideaware_stream_t; /* hipStream_t */
+
+/* ---- PyTorch pluggable allocator entry points ------------------------------------------ */
+
+/* sideaware.cu:1320.  Null on out-of-memory (PyTorch turns that into its OOM exception).
+ * Requests of at least the large threshold (8 MiB unless changed) get a region of their own,
+ * aligned to 2 MiB; smaller ones a 512 B-aligned block of a pooled size class. */
+void* sideaware_malloc_auto(size_t size, int device, sideaware_stream_t stream);
+/* sideaware.cu:1343.  Null is ignored; a pointer this library did not hand out goes to hipFree. */
+void sideaware_free_auto(void* ptr, size_t size, int device, sideaware_stream_t stream);
+
+/* ---- direct allocation (example_llmc_rope.cu:265,314) ---------------------------------- */
+
+/* sideaware.cu:1292 / :1301.  Device-synchronising; always a 2 MiB-aligned region. */
+int sideaware_malloc(void** dev_ptr, size_t size);
+int sideaware_free(void* ptr);
+/* sideaware.cu:1280 / :1286.  Stream-ordered: the block may be reused by later work on `stream`
+ * at once, and by another stream only after `stream` has been waited for. */
+int sideaware_malloc_async(void** dev_ptr, size_t size, sideaware_stream_t stream);
+int sideaware_free_async(void* ptr, sideaware_stream_t stream);
+/* sideaware.cu:1307.  Returns every cached byte to the driver; returns the byte count. */
+size_t sideaware_release_unused(void);
+
+/* ---- kernels ----------------------------------------------------------------------------- */
+
+/* sideaware.cu:1460 / :1421.  Registers an op header (text; copied) and returns its id.
+ * Empty or null selects id 0, the built-in copy.  The same text always returns the same id.
+ * Compilation happens on first launch unless `precompile`.  `default_num_groups` <= 0 lets
+ * the library choose the number of 256-thread workgroups per CU from the kernel's occupancy. */
+int sideaware_create_kernel(const char* header);
+int sideaware_create_kernel_advanced(const char* header, bool precompile, int default_num_groups);
+
+/* sideaware.cu:1358.  num_bytes is the length of the array whose elements are the wider of
+ * (i0, o0); it and the in0/out0 pointers must be multiples of 16.  parallel_groups > 0 fixes
+ * the workgroups per CU, forced_per_side > 0 the CUs used per XCD.  Returns at once when
+ * num_bytes is 0 or both in0 and out0 are null. */
+void sideaware_elementwise(int kernel_id, size_t num_bytes,
+                           void* out0, void* out1, void* out2, void* out3,
+                           const void* in0, const void* in1, const void* in2, const void* in3,
+                           void* sideband_memory, int sideband_value,
+                           int parallel_groups, int forced_per_side,
+                           int device, sideaware_stream_t stream);
+/* sideaware.cu:1410 */
+void sideaware_one_to_one(int kernel_id, size_t num_bytes, void* out0, const void* in0,
+                          int device, sideaware_stream_t stream);
+/* sideaware.cu:1414 */
+void sideaware_memcpy(void* out, const void* in, size_t num_bytes, int device, sideaware_stream_t stream);
+
+/* ---- configuration (sideaware.cu:1467-1487) -------------------------------------------- */
+
+void sideaware_compression(bool enable);              /* accepted, no effect: no such memory type here */
+void sideaware_alloc_threshold(size_t threshold);     /* large/small boundary of malloc_auto */
+void sideaware_prealloc_config(int extra_required, int extra_alloc); /* accepted, no effect: nothing is pre-mapped */
+void sideaware_free_mapped_thresholds(size_t start_threshold, size_t end_threshold);
+                                                      /* cached large bytes above `start` are trimmed to `end` on a miss */
+void sideaware_write_sass(const char* filename);      /* append the gfx950 ISA of every later compile to this file */
+
+/* ---- queries (sideaware.cu:1492-1522) ---------------------------------------------------- */
+
+/* One byte per CU-sized workgroup slot i of a one-workgroup-per-CU launch:
+ * (rank within its XCD << 3) | XCD, the XCD as read from the hardware at start-up. */
+void sideaware_fill_side_index(unsigned char* gpu_array);   /* copies num_sms bytes device-to-device */
+const char* sideaware_gpu_side_index(void);                 /* device copy of that table */
+const char* sideaware_cpu_side_index(void);                 /* host copy */
+/* int[5]: { CUs, CUs on XCD 0, CUs on XCD 1, fewest CUs on any XCD, stripe hash | 1<<21 }.
+ * The hash has the address bits that choose the owning XCD of a byte in a 2 MiB-aligned region. */
+const int* sideaware_sm_side_summary(void);
+int sideaware_num_sms(void);
+int sideaware_num_sm_side0(void);
+int sideaware_num_sm_side1(void);
+int sideaware_min_sm_per_side(void);
+int sideaware_hash_mask(void);
+
+/* ---- additions (no counterpart in the reference) ---------------------------------------- */
+
+int sideaware_num_xcds(void);
+/* 1 when the start-up probe found workgroup i of a launch on XCD i % num_xcds. */
+int sideaware_xcd_dealing_verified(void);
+/* Text of the most recent failure on any thread ("" if none). */
+const char* sideaware_last_error(void);
+void sideaware_clear_error(void);
+/* Compiles header + template for gfx950 without touching a device. variant 0 = 32-bit indices
+ * and 2 MiB-aligned base, 1 = 64-bit indices and any base.  Returns 0 on success; the compiler
+ * log (possibly empty) is copied to `log`. */
+int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity);
+/* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */
+const char* sideaware_kernel_source(void);
+const char* sideaware_memcpy_header(void);
+/* The configuration block the host would prepend for `variant` with the current tuning. */
+const char* sideaware_config_block(int variant);
+/* out[0..3] = { VGPRs, SGPRs, workgroups per CU by occupancy, default workgroups per CU }
+ * of a compiled kernel; compiles it if needed.  Returns 0 on success. */
+int sideaware_kernel_info(int kernel_id, int variant, int* out);
+/* Pool counters, in the order of struct PoolStats (pool.h); returns the number written. */
+int sideaware_alloc_stats(unsigned long long* out, int capacity);
+/* Tuning knobs: "stripe_bytes", "nt_store", "groups_cap", "wg_threads", "shrink_grid".
+ * Setting one drops every compiled kernel.  Returns 0 if the key is known. */
+int sideaware_tune(const char* key, long long value);
+long long sideaware_tune_get(const char* key);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SIDEAWARE_H */

@@ -1,0 +1,83 @@
+#include "hip_backing.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+
+namespace sideaware {
+
+namespace {
+struct DeviceGuard {
+    int prev = -1;
+    bool switched = false;
+    explicit DeviceGuard(int want) {
+        if (hipGetDevice(&prev) == hipSuccess && prev != want) {
+            switched = hipSetDevice(want) == hipSuccess;
+        }
+    }
+    ~DeviceGuard() {
+        if (switched) (void)hipSetDevice(prev);
+    }
+};
+}  // namespace
+
+// hipMalloc returns 2 MiB-aligned addresses for requests of this size on current ROCm, but
+// nothing promises it, so a misaligned answer is replaced by an over-sized one whose aligned
+// interior is handed out instead.
+void* HipBacking::acquire(size_t bytes) {
+    DeviceGuard g(device_);
+    void* raw = nullptr;
+    if (hipMalloc(&raw, bytes) != hipSuccess) {
+        (void)hipGetLastError();      // an out-of-memory answer must not poison later calls
+        return nullptr;
+    }
+    void* aligned = raw;
+    if ((uintptr_t)raw % kRegionAlign != 0) {
+        (void)hipFree(raw);
+        raw = nullptr;
+        if (hipMalloc(&raw, bytes + kRegionAlign) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        aligned = (void*)(((uintptr_t)raw + kRegionAlign - 1) / kRegionAlign * kRegionAlign);
+    }
+    std::lock_guard<std::mutex> lk(mu_);
+    raw_of_[aligned] = raw;
+    return aligned;
+}
+
+void HipBacking::release(void* ptr, size_t) {
+    void* raw = ptr;
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        auto it = raw_of_.find(ptr);
+        if (it != raw_of_.end()) {
+            raw = it->second;
+            raw_of_.erase(it);
+        }
+    }
+    DeviceGuard g(device_);
+    if (hipFree(raw) != hipSuccess) {
+        std::fprintf(stderr, "sideaware: hipFree(%p) failed: %s\n", raw, hipGetErrorString(hipGetLastError()));
+    }
+}
+
+void HipBacking::sync_device() {
+    DeviceGuard g(device_);
+    (void)hipDeviceSynchronize();
+}
+
+void HipBacking::sync_stream(void* stream) {
+    DeviceGuard g(device_);
+    (void)hipStreamSynchronize((hipStream_t)stream);
+}
+
+int HipBacking::free_foreign(void* ptr, void* stream) {
+    DeviceGuard g(device_);
+    (void)stream;
+    hipError_t e = hipFree(ptr);
+    if (e != hipSuccess) (void)hipGetLastError();
+    return (int)e;
+}
+
+}  // namespace sideaware

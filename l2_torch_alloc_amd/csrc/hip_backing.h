@@ -1,0 +1,28 @@
+// The pool's backing store on a real device: plain hipMalloc / hipFree.
+#pragma once
+
+#include <mutex>
+#include <unordered_map>
+
+#include "pool.h"
+
+namespace sideaware {
+
+class HipBacking final : public Backing {
+public:
+    explicit HipBacking(int device) : device_(device) {}
+    void* acquire(size_t bytes) override;
+    void release(void* ptr, size_t bytes) override;
+    void sync_device() override;
+    void sync_stream(void* stream) override;
+    int free_foreign(void* ptr, void* stream) override;
+
+private:
+    int device_;
+    std::mutex mu_;
+    // aligned pointer handed to the pool -> pointer hipMalloc returned (they differ only when
+    // the runtime did not return a 2 MiB-aligned address by itself)
+    std::unordered_map<void*, void*> raw_of_;
+};
+
+}  // namespace sideaware

@@ -1,0 +1,149 @@
+// Device-memory pool behind the sideaware_* allocation entry points.
+//
+// The reference keeps two pools of 2 MiB physical pages (one per H100 L2 side), maps them so
+// that virtual-address bit 21 predicts the side, and reuses freed blocks of exactly the same
+// rounded size (sideaware.cu:934-1273).  On MI355X there are no sides to sort pages by: the
+// eight XCDs reach all of HBM through the memory-side Infinity Cache, and which XCD touches
+// which byte is decided by the kernels' workgroup -> stripe map.  What the kernels need from
+// the allocator is therefore only a *phase guarantee*: every large region starts on a
+// kRegionAlign (2 MiB) boundary, a whole number of XCD stripe periods, so offset o of any two
+// regions falls in the same XCD's stripe.  The pool delivers that, plus the reference's
+// caching behaviour:
+//
+//   large  (size >= threshold): dedicated region, size rounded up to 2 MiB, exact-size LIFO
+//          reuse cache, trimmed back to the backing store when it outgrows the thresholds,
+//          and the reference's four-step out-of-memory ladder (sideaware.cu:1233-1252);
+//   small  (size <  threshold): 512 B-granular size classes carved from slabs, so the common
+//          small request never reaches the driver (the reference forwards these to
+//          cudaMallocAsync, sideaware.cu:1326-1339).
+//
+// All device interaction goes through the Backing interface, so every policy decision in here
+// runs on a CPU with a fake backing (tests/test_pool.py).  One mutex guards all state: the
+// PyTorch caching layer may call in from several threads.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace sideaware {
+
+constexpr size_t kRegionAlign = 2ull << 20;      // alignment and rounding of large regions
+constexpr size_t kSmallGranule = 512;            // alignment and minimum size of small blocks
+constexpr size_t kMaxSlabBytes = 64ull << 20;
+
+// Where the bytes come from.  The HIP implementation lives in hip_backing.cpp.
+class Backing {
+public:
+    virtual ~Backing() = default;
+    // Returns a pointer aligned to kRegionAlign, or nullptr when the device is out of memory.
+    virtual void* acquire(size_t bytes) = 0;
+    virtual void release(void* ptr, size_t bytes) = 0;
+    // Block until every stream of the device is idle (before memory goes back to the driver).
+    virtual void sync_device() = 0;
+    // Block until `stream` is idle (before a block moves to another stream).
+    virtual void sync_stream(void* stream) = 0;
+    // A pointer the pool never handed out: forward to the runtime's own free.
+    virtual int free_foreign(void* ptr, void* stream) = 0;
+};
+
+struct PoolStats {
+    uint64_t large_hits = 0;        // large requests served from the reuse cache
+    uint64_t large_misses = 0;      // large requests that went to the backing store
+    uint64_t small_hits = 0;        // small requests served from a class free list
+    uint64_t small_carves = 0;      // small requests carved from a slab's untouched tail
+    uint64_t slabs_acquired = 0;
+    uint64_t backing_acquires = 0;
+    uint64_t backing_releases = 0;
+    uint64_t stream_syncs = 0;
+    uint64_t device_syncs = 0;
+    uint64_t trims = 0;             // threshold-driven trims of the large cache
+    uint64_t ladder_retries = 0;    // times a request needed step 3 or 4 of the ladder
+    uint64_t failures = 0;          // requests that returned nullptr
+    uint64_t foreign_frees = 0;
+    uint64_t bytes_live = 0;        // rounded bytes in blocks currently handed out
+    uint64_t bytes_cached_large = 0;
+    uint64_t bytes_cached_small = 0;
+    uint64_t bytes_reserved = 0;    // everything held from the backing store
+    uint64_t peak_reserved = 0;
+};
+constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
+
+class Pool {
+public:
+    explicit Pool(Backing* backing);
+    ~Pool();
+
+    // Configuration (the reference's file-static knobs, sideaware.cu:419-423).
+    void set_large_threshold(size_t bytes);
+    size_t large_threshold() const { return large_threshold_; }
+    void set_trim_thresholds(size_t start_bytes, size_t end_bytes);
+
+    // always_large: the reference's direct C entry points (sideaware_malloc and friends,
+    // sideaware.cu:1280-1305) never take the small path.
+    void* allocate(size_t bytes, void* stream, bool always_large);
+    // Returns 0 on success, or the backing's code for a pointer the pool does not own.
+    int deallocate(void* ptr, void* stream);
+
+    // Gives every cached byte back to the backing store; returns how many.
+    size_t release_unused();
+
+    PoolStats stats();
+    // For the property tests: true when `ptr` is a live block of this pool.
+    bool owns_live(void* ptr);
+
+    static size_t round_large(size_t bytes);
+    static size_t small_class_size(size_t bytes);   // rounded size of a small request
+    static int small_class_index(size_t bytes);
+
+private:
+    struct LargeBlock {
+        void* ptr = nullptr;
+        size_t bytes = 0;          // rounded
+        void* last_stream = nullptr;
+    };
+    struct Slab {
+        char* base = nullptr;
+        size_t bytes = 0;
+        size_t block = 0;          // class size
+        uint32_t capacity = 0;     // blocks in the slab
+        uint32_t carved = 0;       // blocks ever handed out from the bump pointer
+        uint32_t live = 0;
+        std::vector<uint8_t> in_use;   // one flag per block: catches double frees
+    };
+    struct FreeSmall {
+        void* ptr;
+        void* stream;
+    };
+    struct SmallClass {
+        std::vector<FreeSmall> free;
+        std::vector<Slab*> slabs;
+        Slab* bump = nullptr;      // slab still holding never-used blocks
+    };
+
+    void* allocate_large_locked(size_t bytes, void* stream);
+    void* allocate_small_locked(size_t bytes, void* stream);
+    void* acquire_large_locked(size_t rounded, void* stream);
+    Slab* new_slab_locked(size_t block);
+    size_t trim_large_locked(size_t down_to);
+    size_t release_empty_slabs_locked();
+    void note_reserved(int64_t delta);
+
+    Backing* backing_;
+    std::mutex mu_;
+    size_t large_threshold_ = 8ull << 20;
+    size_t trim_start_ = 16ull << 30;
+    size_t trim_end_ = 2ull << 30;
+
+    std::unordered_map<size_t, std::vector<LargeBlock>> large_cache_;  // rounded size -> LIFO
+    std::unordered_map<void*, LargeBlock> large_live_;
+    std::vector<SmallClass> small_;                                    // class index -> state
+    std::unordered_map<uintptr_t, Slab*> slab_by_page_;                // addr >> 21 -> slab
+    std::vector<std::unique_ptr<Slab>> slab_store_;
+    PoolStats st_;
+};
+
+}  // namespace sideaware

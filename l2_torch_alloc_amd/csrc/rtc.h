@@ -1,0 +1,27 @@
+// Run-time compilation of kernel source for gfx950 with hipRTC, and the small services around
+// it: in-memory compatibility headers, an on-disk cache of code objects, and an ISA dump.
+// Takes the place of the reference's NVRTC -> cubin step (sideaware.cu:523-607).
+#pragma once
+
+#include <string>
+#include <vector>
+
+namespace sideaware {
+
+struct CompileResult {
+    bool ok = false;
+    bool from_disk_cache = false;
+    std::vector<char> code;     // gfx950 code object
+    std::string log;            // compiler diagnostics (warnings on success, errors on failure)
+};
+
+// Compiles `source` (one translation unit, already holding the configuration block, the user's
+// header and the kernel template).  Needs no GPU: hipRTC cross-compiles.
+CompileResult compile_for_gfx950(const std::string& source, const char* arch = "gfx950");
+
+// Where every later successful compile appends its disassembly ("" = nowhere).  The reference
+// dumps SASS through cuobjdump (sideaware.cu:572-599); here it is the gfx950 ISA of the code
+// object just built, through the ROCm llvm-objdump.
+void set_isa_dump_file(const std::string& filename);
+
+}  // namespace sideaware

@@ -1,0 +1,98 @@
+// Appended after the kernel template: runs the whole grid on the CPU, lane by lane, and checks
+// the result.  stdin carries one case per line: "grid num_vectors base_offset_bytes".
+//
+// Every array is a posix_memalign block of exactly the bytes it needs, 2 MiB-aligned and then
+// shifted by base_offset, so a lane that reads or writes past the end trips AddressSanitizer
+// and a write before the start is caught by the sentinel bytes in front.
+//
+// SA_CASE_INCREMENT: the op adds 1 to i0 in place (out0 aliases in0), so "each vector is
+//   visited exactly once" is the same as "each element ends at seed + 1".
+// SA_CASE_MIXED: four arrays of different element widths; checks that narrow and wide arrays are
+//   addressed with the same element index and that element_idx counts elements of the array.
+#include <cstdio>
+#include <cstdlib>
+
+static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3* o3,
+                     const vi0* i0, const vi1* i1, const vi2* i2, const vi3* i3, int* mem, int val) {
+    gridDim = {grid, 1, 1};
+    blockDim = {SA_WG_THREADS, 1, 1};
+    for (unsigned b = 0; b < grid; b++) {
+        for (unsigned t = 0; t < SA_WG_THREADS; t++) {
+            blockIdx = {b, 0, 0};
+            threadIdx = {t, 0, 0};
+            sideaware_elementwise(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val);
+        }
+    }
+}
+
+struct Arena {
+    char* block = nullptr;
+    char* data = nullptr;
+    size_t off = 0;
+    Arena(size_t offset, size_t bytes) : off(offset) {
+        if (posix_memalign((void**)&block, 2u << 20, offset + bytes + (bytes == 0)) != 0) std::abort();
+        std::memset(block, 0xAB, offset);
+        data = block + offset;
+    }
+    bool sentinel_ok() const {
+        for (size_t i = 0; i < off; i++) if ((unsigned char)block[i] != 0xAB) return false;
+        return true;
+    }
+    ~Arena() { std::free(block); }
+};
+
+#if defined(SA_CASE_INCREMENT)
+static int run_case(unsigned grid, long long nv, size_t off) {
+    const size_t n = (size_t)nv * vec_size;
+    Arena a(off, n * sizeof(int));
+    int* x = (int*)a.data;
+    for (size_t i = 0; i < n; i++) x[i] = (int)(i * 7u + 3u);
+    run_grid(grid, (size_type)nv, (vo0*)x, nullptr, nullptr, nullptr, (const vi0*)x, nullptr, nullptr, nullptr,
+             nullptr, 0);
+    int bad = a.sentinel_ok() ? 0 : 1;
+    for (size_t i = 0; i < n; i++) bad += (x[i] != (int)(i * 7u + 3u) + 1);
+    return bad;
+}
+#elif defined(SA_CASE_MIXED)
+static int run_case(unsigned grid, long long nv, size_t off) {
+    const size_t n = (size_t)nv * vec_size;
+    // only o0's array (the widest of i0/o0) is shifted by `off`; the narrower ones shift in proportion
+    Arena f_out(off, n * sizeof(float)), s_out(off / 2, n * sizeof(short)), idx_out(off, n * sizeof(int));
+    Arena s_in(off / 2, n * sizeof(short)), f_in(off, n * sizeof(float));
+    short* si = (short*)s_in.data;
+    float* fi = (float*)f_in.data;
+    for (size_t i = 0; i < n; i++) { si[i] = (short)(i % 1000); fi[i] = (float)(i % 77) * 0.5f; }
+    std::memset(f_out.data, 0, n * sizeof(float));
+    std::memset(s_out.data, 0, n * sizeof(short));
+    std::memset(idx_out.data, 0xff, n * sizeof(int));
+    run_grid(grid, (size_type)nv, (vo0*)f_out.data, (vo1*)s_out.data, (vo2*)idx_out.data, nullptr,
+             (const vi0*)si, (const vi1*)fi, nullptr, nullptr, nullptr, 5);
+    int bad = 0;
+    bad += !f_out.sentinel_ok() + !s_out.sentinel_ok() + !idx_out.sentinel_ok();
+    for (size_t i = 0; i < n; i++) {
+        bad += (((float*)f_out.data)[i] != (float)si[i] + fi[i]);
+        bad += (((short*)s_out.data)[i] != (short)(fi[i] * 10.0f + 5.0f));
+        bad += (((int*)idx_out.data)[i] != (int)i);
+    }
+    return bad;
+}
+#else
+#error "define SA_CASE_INCREMENT or SA_CASE_MIXED"
+#endif
+
+int main() {
+    unsigned grid;
+    long long nv;
+    size_t off;
+    int cases = 0, failed = 0;
+    while (std::scanf("%u %lld %zu", &grid, &nv, &off) == 3) {
+        cases++;
+        int bad = run_case(grid, nv, off);
+        if (bad) {
+            failed++;
+            std::printf("FAIL grid=%u nv=%lld off=%zu: %d bad elements\n", grid, nv, off, bad);
+        }
+    }
+    std::printf("cases=%d failed=%d\n", cases, failed);
+    return failed ? 1 : 0;
+}

@@ -1,0 +1,138 @@
+"""Runs the shipped kernel template on the CPU, lane by lane, under AddressSanitizer.
+
+The text comes out of the built library (``sideaware_kernel_source`` / ``sideaware_config_block``),
+so what is checked is exactly what hipRTC compiles on the GPU box.  For each compile-time
+configuration (index width, UNROLLED, ownership stripe, traversal order) a small driver is built
+with the ROCm clang as plain host C++ and fed many (grid, length, base offset) cases: the
+workgroup -> tile map must visit every 16-byte vector exactly once, never touch a byte outside
+the arrays, and do so for any grid size, which is the property the reference could not offer
+(its map skips data unless exactly one block runs per SM, sideaware.cu:211-212).
+"""
+import ctypes
+import os
+import random
+import subprocess
+
+import pytest
+
+from l2_torch_alloc_amd import build as sa_build
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+NATIVE = os.path.join(HERE, "native")
+CLANG = os.path.join(sa_build.rocm_root(), "lib", "llvm", "bin", "clang++")
+
+INCREMENT_HEADER = """
+typedef int o0;
+typedef int i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = %(reverse)s;
+constexpr bool input_evict[4] = {true, false, false, false};
+%(unrolled)s
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = in0 + 1;
+}
+"""
+
+MIXED_HEADER = """
+typedef float o0;
+typedef short o1;
+typedef int   o2;
+typedef short i0;
+typedef float i1;
+struct unused {};
+typedef unused o3, i2, i3;
+constexpr bool reverse_order = %(reverse)s;
+constexpr bool input_evict[4] = {true, true, false, false};
+%(unrolled)s
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = (float)in0 + in1;
+    out1 = (short)(in1 * 10.0f + (float)sideband);
+    out2 = (int)element_idx;
+}
+"""
+
+
+@pytest.fixture(scope="module")
+def lib():
+    path = sa_build.build_library(force=False)
+    L = ctypes.CDLL(path)
+    L.sideaware_kernel_source.restype = ctypes.c_char_p
+    L.sideaware_config_block.restype = ctypes.c_char_p
+    L.sideaware_config_block.argtypes = [ctypes.c_int]
+    L.sideaware_tune.argtypes = [ctypes.c_char_p, ctypes.c_longlong]
+    return L
+
+
+def build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse):
+    assert lib.sideaware_tune(b"stripe_bytes", stripe) == 0
+    config = lib.sideaware_config_block(variant).decode()
+    template = lib.sideaware_kernel_source().decode()
+    header = (INCREMENT_HEADER if case == "INCREMENT" else MIXED_HEADER) % {
+        "reverse": "true" if reverse else "false",
+        "unrolled": "" if unrolled is None else "#define UNROLLED %d" % unrolled,
+    }
+    tu = "\n".join([
+        '#include "%s"' % os.path.join(NATIVE, "kernel_cpu_prelude.h"),
+        config, header, template,
+        "#define SA_CASE_%s 1" % case,
+        '#include "%s"' % os.path.join(NATIVE, "kernel_cpu_driver.h"),
+    ])
+    src = tmp_path / ("tu_%s_v%d_u%s_s%d_r%d.cpp" % (case, variant, unrolled, stripe, reverse))
+    exe = str(src)[:-4]
+    src.write_text(tu)
+    cmd = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
+           "-fno-sanitize-recover=undefined", "-Wno-unused-value", str(src), "-o", exe]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    return exe
+
+
+def cases_for(variant, unrolled, rng):
+    tile = 256 * (unrolled or 4)
+    lengths = {0, 1, 2, 15, 16, 255, 256, 257, tile - 1, tile, tile + 1, 2 * tile, 8 * tile, 8 * tile + 1,
+               64 * tile - 1, 777, 3108 // 4}      # 777: the reference's (4, 777) fp32 case is 777 vectors
+    lengths |= {rng.randrange(0, 70 * tile) for _ in range(40)}
+    # every residue class of the tail for one tile count, sampled
+    lengths |= {5 * tile + r for r in rng.sample(range(tile), 24)}
+    grids = [8, 16, 24, 56, 8 * 37, 2048]
+    offsets = [0] if variant == 0 else [0, 16, 4096, 16384 + 32, 3 * 65536 + 4096 + 48, (2 << 20) - 16]
+    out = []
+    for n in sorted(lengths):
+        for g in rng.sample(grids, 2):
+            for off in rng.sample(offsets, min(2, len(offsets))):
+                out.append((g, n, off))
+    return out
+
+
+CONFIGS = [
+    # case, variant, UNROLLED (None = template default), stripe bytes, reverse_order
+    ("INCREMENT", 0, None, 16384, False),
+    ("INCREMENT", 1, None, 16384, False),
+    ("INCREMENT", 0, 1, 4096, True),
+    ("INCREMENT", 1, 2, 65536, True),
+    ("INCREMENT", 1, 3, 16384, False),      # tile is not a power of two
+    ("INCREMENT", 0, 8, 4096, False),       # tile larger than the stripe
+    ("INCREMENT", 1, 4, 262144, True),      # largest stripe with the 2 MiB phase guarantee
+    ("MIXED", 0, None, 16384, False),
+    ("MIXED", 1, 2, 4096, True),
+]
+
+
+@pytest.mark.parametrize("case,variant,unrolled,stripe,reverse", CONFIGS)
+def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, stripe, reverse):
+    if not os.path.exists(CLANG):
+        pytest.skip("ROCm clang++ not found")
+    exe = build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse)
+    rng = random.Random(hash((case, variant, unrolled, stripe, reverse)) & 0xffff)
+    cases = cases_for(variant, unrolled, rng)
+    if case == "MIXED":
+        cases = [(g, n, off - off % 64) for (g, n, off) in cases]   # halves of the offset stay 16 B-aligned
+    text = "".join("%d %d %d\n" % c for c in cases)
+    proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
+                          env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
+    assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
+    assert "cases=%d failed=0" % len(cases) in proc.stdout
