@@ -1,0 +1,155 @@
+"""Op headers for the run-time compiled elementwise kernel.
+
+An op header is the text the caller hands to ``sideaware_create_kernel``: element types
+``o0..o3`` / ``i0..i3``, ``reverse_order``, ``input_evict`` and ``elementwise_op``, plus optional
+hooks.  The contract is the reference's (``sideaware.cu:33-48``, ``kernel_rope.cuh:1-60``,
+``test.py:191-216``); the generators below bake the problem shape into the text the way the
+reference's RoPE header does with its ``constexpr int T / n_head / head_dim``
+(``kernel_rope.cuh:21-27``), but for any shape, for bf16 storage and for separate q / k tensors.
+
+Arithmetic follows the llm.c formula (``example_llmc_rope.cu:70-81``, ``kernel_rope.cuh:29-40``):
+``out = (x_re*c - x_im*s, x_re*s + x_im*c)`` in fp32, each product rounded before the add (the
+library compiles with contraction off), so fp32 results are bit-identical to a CPU that does not
+fuse.  bf16 storage widens exactly, computes in fp32 and rounds to nearest even on store.
+"""
+from __future__ import annotations
+
+_UNUSED = "struct unused {};\n"
+
+
+def _evict(flags) -> str:
+    flags = list(flags) + [False] * (4 - len(flags))
+    return "constexpr bool input_evict[4] = {%s};\n" % ", ".join("true" if f else "false" for f in flags)
+
+
+def memcpy_header() -> bytes:
+    """The built-in copy (kernel id 0), spelled out: 4-byte elements, input read once."""
+    return (
+        "typedef int o0;\ntypedef int i0;\n" + _UNUSED +
+        "typedef unused o1, o2, o3, i1, i2, i3;\n"
+        "constexpr bool reverse_order = false;\n" + _evict([True]) +
+        "__device__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {\n"
+        "    out0 = in0;\n}\n"
+    ).encode()
+
+
+_ROPE_TYPES = {
+    # storage dtype -> (declarations, element type of one (re, im) pair, widen, narrow)
+    "fp32": ("", "float2", "%s", "%s"),
+    "bf16": ("struct sa_bf16_pair { __bf16 x, y; };\n", "sa_bf16_pair", "(float)%s", "(__bf16)(%s)"),
+}
+
+
+def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
+                layout: str = "qkv", backward: bool = False, unrolled: int | None = None,
+                reverse_order: bool = False) -> bytes:
+    """RoPE forward (or backward) in place or out of place.
+
+    layout "qkv":   one tensor (B, T, n_q + 2*n_kv, head_dim); q and k heads are rotated, the
+                    trailing n_kv value heads are skipped (neither read nor written), which is
+                    the reference's packed layout (``kernel_rope.cuh:42-60``) with GQA head counts.
+    layout "heads": one tensor (B, T, n_q, head_dim), every head rotated (``n_kv`` ignored):
+                    separate q and k tensors take one launch each.
+
+    in0/out0 is the activation, in1 the fp32 table (T, head_dim/2, 2) of (cos, sin) pairs.
+    ``num_bytes`` at launch is the byte size of the activation tensor.
+    """
+    if dtype not in _ROPE_TYPES:
+        raise ValueError("dtype must be 'fp32' or 'bf16'")
+    if layout not in ("qkv", "heads"):
+        raise ValueError("layout must be 'qkv' or 'heads'")
+    if head_dim % 2:
+        raise ValueError("head_dim must be even")
+    decl, pair, widen, narrow = _ROPE_TYPES[dtype]
+    pair_bytes = 8 if dtype == "fp32" else 4
+    pairs_per_vec = 16 // pair_bytes
+    half = head_dim // 2
+    if half % pairs_per_vec:
+        raise ValueError("head_dim/2 must be a multiple of %d for %s" % (pairs_per_vec, dtype))
+    total_heads = n_q + 2 * n_kv if layout == "qkv" else n_q
+    rotated_heads = n_q + n_kv if layout == "qkv" else n_q
+    sign_a, sign_b = ("+", "-") if backward else ("-", "+")
+
+    lines = [decl]
+    lines.append("typedef %s o0;\ntypedef %s i0;\ntypedef float2 i1;\n" % (pair, pair))
+    lines.append(_UNUSED + "typedef unused o1, o2, o3, i2, i3;\n")
+    if unrolled is not None:
+        lines.append("#define UNROLLED %d\n" % unrolled)
+    lines.append("constexpr bool reverse_order = %s;\n" % ("true" if reverse_order else "false"))
+    lines.append(_evict([True, False]))      # activations stream; the table is re-read and stays cached
+    lines.append(
+        "constexpr int rope_T = %d;\n"
+        "constexpr int rope_half = %d;          // pairs per head\n"
+        "constexpr int rope_heads = %d;         // heads per token in this tensor\n"
+        "constexpr int rope_rotated = %d;       // leading heads that are rotated\n"
+        % (T, half, total_heads, rotated_heads))
+    lines.append(
+        "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {\n"
+        "    const float x_re = %s, x_im = %s;\n"
+        "    const float c = in1.x, s = in1.y;\n"
+        "    const float y_re = x_re * c %s x_im * s;\n"
+        "    const float y_im = x_im * c %s x_re * s;\n"
+        "    out0.x = %s;\n"
+        "    out0.y = %s;\n"
+        "}\n" % (widen % "in0.x", widen % "in0.y", sign_a, sign_b, narrow % "y_re", narrow % "y_im"))
+    # A 16-byte vector holds pairs_per_vec consecutive pairs of one head of one token, so one
+    # decode serves the whole vector: the table row of the token, at the head-local pair.
+    lines.append(
+        "#define CUSTOM_IDX_FUNC\n"
+        "__device__ __forceinline__ bool indexing(size_type vec_idx, int vec_size,\n"
+        "                         size_type &idx_i0, size_type &idx_i1,\n"
+        "                         size_type &idx_i2, size_type &idx_i3, int* mem, int val) {\n"
+        "    const size_type pair = vec_idx * vec_size;\n"
+        "    const int head = (int)((pair / rope_half) % rope_heads);\n"
+        "    const int token = (int)((pair / ((size_type)rope_heads * rope_half)) % rope_T);\n"
+        "    const int local = (int)(pair % rope_half);\n"
+        "    idx_i0 = vec_idx;\n"
+        "    idx_i1 = (size_type)((token * rope_half + local) / vec_size);\n"
+        "    idx_i2 = 0;\n"
+        "    idx_i3 = 0;\n"
+        "    return head >= rope_rotated;\n"
+        "}\n")
+    return "".join(lines).encode()
+
+
+def scale_bias_bf16_header(unrolled: int | None = None) -> bytes:
+    """bf16 ``y = x*scale + bias``; scale and bias are two fp32 values read from the sideband
+    pointer at launch, so one compiled kernel serves every (scale, bias)."""
+    lines = ["typedef __bf16 o0;\ntypedef __bf16 i0;\n", _UNUSED, "typedef unused o1, o2, o3, i1, i2, i3;\n"]
+    if unrolled is not None:
+        lines.append("#define UNROLLED %d\n" % unrolled)
+    lines.append("constexpr bool reverse_order = false;\n" + _evict([True]))
+    lines.append(
+        "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}\n"
+        "#define CUSTOM_VECTOR_OP\n"
+        "__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size,\n"
+        "                          o0 *out0, o1 *out1, o2 *out2, o3 *out3,\n"
+        "                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,\n"
+        "                          int* sideband_memory, int sideband_value) {\n"
+        "    const float scale = ((const float*)sideband_memory)[0];\n"
+        "    const float bias  = ((const float*)sideband_memory)[1];\n"
+        "    #pragma unroll\n"
+        "    for (int i = 0; i < vec_size; i++) {\n"
+        "        const float p = (float)in0[i] * scale;\n"
+        "        out0[i] = (__bf16)(p + bias);\n"
+        "    }\n"
+        "}\n")
+    return "".join(lines).encode()
+
+
+def fill_header() -> bytes:
+    """Writes the 32-bit sideband value to every element: an output-only op (no in0)."""
+    return (
+        "typedef int o0;\n" + _UNUSED + "typedef unused o1, o2, o3, i0, i1, i2, i3;\n"
+        "constexpr bool reverse_order = false;\n" + _evict([]) +
+        "__device__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {\n"
+        "    out0 = sideband;\n}\n"
+    ).encode()

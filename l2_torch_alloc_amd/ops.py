@@ -1,0 +1,111 @@
+"""Ready-made ops on top of ``torch.ops.sideaware.elementwise``: RoPE (llm.c formula), bf16
+scale+bias and fill.  Each builds its op header once per shape (``headers.py``), registers it with
+the library and launches through the same custom op a user-written header would use.
+
+The frequency table is an *input*: build it on the host with ``freqs_cis_table`` (the llm.c
+formula, ``example_llmc_rope.cu:19-52``) or bring your own, as (T, head_dim) fp32 with cos at
+even and sin at odd columns.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import headers, wrapper
+
+_kernel_ids: Dict[Tuple, int] = {}
+
+
+def _kernel(key: Tuple, make_header) -> int:
+    kid = _kernel_ids.get(key)
+    if kid is None:
+        kid = wrapper.sideaware_create_kernel(make_header())
+        _kernel_ids[key] = kid
+    return kid
+
+
+def freqs_cis_table(head_dim: int, end: int, theta: float, use_scaled: bool = False) -> torch.Tensor:
+    """(end, head_dim) fp32 table on the host: [t, 2i] = cos(t*f_i), [t, 2i+1] = sin(t*f_i),
+    f_i = theta^(-2i/head_dim) in fp32, optionally with the Llama-3.1 wavelength rescaling
+    (``example_llmc_rope.cu:25-43``).  Built with torch CPU ops in fp32."""
+    i = torch.arange(head_dim // 2, dtype=torch.float32)
+    freq = 1.0 / torch.pow(torch.tensor(theta, dtype=torch.float32), (2 * i) / head_dim)
+    if use_scaled:
+        scale_factor, low_factor, high_factor, old_len = 8.0, 1.0, 4.0, 8192.0
+        wavelen = (2.0 * math.pi / freq.double()).float()
+        smooth = (old_len / wavelen - low_factor) / (high_factor - low_factor)
+        blended = (1.0 - smooth) * freq / scale_factor + smooth * freq
+        freq = torch.where(wavelen < old_len / high_factor, freq,
+                           torch.where(wavelen > old_len / low_factor, freq / scale_factor, blended))
+    angle = torch.arange(end, dtype=torch.float32)[:, None] * freq[None, :]
+    table = torch.empty(end, head_dim, dtype=torch.float32)
+    table[:, 0::2] = torch.cos(angle)
+    table[:, 1::2] = torch.sin(angle)
+    return table
+
+
+def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q: int, n_kv: int,
+          layout: str, backward: bool) -> torch.Tensor:
+    assert x.dim() == 4, "activations are (B, T, heads, head_dim)"
+    B, T, heads, head_dim = x.shape
+    if layout == "qkv":
+        assert heads == n_q + 2 * n_kv, "packed QKV needs n_q + 2*n_kv heads"
+    else:
+        n_q, n_kv = heads, 0
+    if x.dtype == torch.float32:
+        dtype = "fp32"
+    elif x.dtype == torch.bfloat16:
+        dtype = "bf16"
+    else:
+        raise TypeError("RoPE storage is float32 or bfloat16")
+    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    if out is None:
+        out = x
+    assert out.shape == x.shape and out.dtype == x.dtype
+    if layout == "qkv" and out.data_ptr() != x.data_ptr():
+        # value heads are skipped by the kernel (neither read nor written): out of place they
+        # have to be carried over by a copy first
+        torch.ops.sideaware.memcpy(out, x)
+    key = ("rope", T, n_q, n_kv, head_dim, dtype, layout, backward)
+    kid = _kernel(key, lambda: headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout, backward))
+    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+    return out
+
+
+def rope_forward_qkv(x, freqs, n_q: int, n_kv: int, out=None):
+    """Packed (B, T, n_q + 2*n_kv, head_dim): rotates q and k heads, leaves v heads alone.
+    In place unless ``out`` is given."""
+    return _rope(x, freqs, out, n_q, n_kv, "qkv", False)
+
+
+def rope_backward_qkv(dout, freqs, n_q: int, n_kv: int, out=None):
+    return _rope(dout, freqs, out, n_q, n_kv, "qkv", True)
+
+
+def rope_forward_heads(x, freqs, out=None):
+    """(B, T, heads, head_dim), every head rotated: one call per separate q or k tensor."""
+    return _rope(x, freqs, out, 0, 0, "heads", False)
+
+
+def rope_backward_heads(dout, freqs, out=None):
+    return _rope(dout, freqs, out, 0, 0, "heads", True)
+
+
+def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[torch.Tensor] = None):
+    """bf16 ``y = x*scale + bias`` in fp32, rounded to nearest even.  ``scale_bias`` is a device
+    tensor of two fp32 values, read by the kernel, so changing them costs no compile."""
+    assert x.dtype == torch.bfloat16 and scale_bias.dtype == torch.float32 and scale_bias.numel() >= 2
+    if out is None:
+        out = torch.empty_like(x)
+    kid = _kernel(("scale_bias_bf16",), headers.scale_bias_bf16_header)
+    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, None, None, None, scale_bias, 0, 0, 0)
+    return out
+
+
+def fill_int32(out: torch.Tensor, value: int):
+    """Writes a 32-bit pattern over ``out`` (byte size a multiple of 16): an output-only op."""
+    kid = _kernel(("fill",), headers.fill_header)
+    torch.ops.sideaware.elementwise(kid, out, None, None, None, None, None, None, None, None, int(value), 0, 0)
+    return out

@@ -25,3 +25,13 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def sa():
+    """The library with PyTorch's device allocations routed through it, as in the reference's
+    scripts (test.py:14-16): installed before the first device allocation of the process, so
+    every tensor any GPU test makes comes from sideaware_malloc_auto."""
+    from l2_torch_alloc_amd import wrapper
+    wrapper.sideaware_init()
+    return wrapper

@@ -76,8 +76,53 @@ static int run_case(unsigned grid, long long nv, size_t off) {
     }
     return bad;
 }
+#elif defined(SA_CASE_ROPE)
+// The op header under test is a generated RoPE header; rope_T / rope_half / rope_heads /
+// rope_rotated come from it.  The activation holds `nv` vectors (any length: a whole number of
+// tokens is not required, the decode must still stay inside the table), the table exactly
+// rope_T * rope_half (cos, sin) pairs, so a wrong table index trips the sanitizer.  Expected
+// values come from nested loops over (row, head, pair) that share no code with `indexing`.
+static float rope_widen(float v) { return v; }
+template<typename Tv> static float rope_widen(Tv v) { return (float)v; }
+static int run_case(unsigned grid, long long nv, size_t off) {
+    typedef decltype(i0().x) scalar;
+    const size_t pairs = (size_t)nv * vec_size;
+    Arena act(off, pairs * sizeof(i0));
+    Arena table(0, (size_t)rope_T * rope_half * sizeof(float2));
+    i0* x = (i0*)act.data;
+    float2* f = (float2*)table.data;
+    for (int t = 0; t < rope_T; t++)
+        for (int d = 0; d < rope_half; d++) {
+            f[(size_t)t * rope_half + d].x = (float)((t * 31 + d * 7) % 64) / 64.0f;
+            f[(size_t)t * rope_half + d].y = (float)((t * 13 + d * 3) % 32) / 32.0f - 0.5f;
+        }
+    for (size_t p = 0; p < pairs; p++) {
+        x[p].x = (scalar)((float)((p * 5) % 33) - 16.0f);
+        x[p].y = (scalar)((float)((p * 11) % 17) - 8.0f);
+    }
+    i0* want = (i0*)std::malloc(pairs * sizeof(i0) + 1);
+    for (size_t p = 0; p < pairs; p++) {
+        size_t row = p / ((size_t)rope_heads * rope_half);      // (batch, token) flattened
+        int head = (int)((p / rope_half) % rope_heads);
+        int d = (int)(p % rope_half);
+        int t = (int)(row % rope_T);
+        want[p] = x[p];
+        if (head < rope_rotated) {
+            float re = rope_widen(x[p].x), im = rope_widen(x[p].y);
+            float c = f[(size_t)t * rope_half + d].x, s = f[(size_t)t * rope_half + d].y;
+            want[p].x = (scalar)(re * c - im * s);
+            want[p].y = (scalar)(im * c + re * s);
+        }
+    }
+    run_grid(grid, (size_type)nv, (vo0*)x, nullptr, nullptr, nullptr, (const vi0*)x, (const vi1*)f, nullptr, nullptr,
+             nullptr, 0);
+    int bad = act.sentinel_ok() ? 0 : 1;
+    for (size_t p = 0; p < pairs; p++) bad += (std::memcmp(&x[p], &want[p], sizeof(i0)) != 0);
+    std::free(want);
+    return bad;
+}
 #else
-#error "define SA_CASE_INCREMENT or SA_CASE_MIXED"
+#error "define SA_CASE_INCREMENT, SA_CASE_MIXED or SA_CASE_ROPE"
 #endif
 
 int main() {

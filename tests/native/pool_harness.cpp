@@ -1,0 +1,103 @@
+// C interface to sideaware::Pool over a fake backing store, for the CPU tests of the allocator's
+// policy: size classes, the exact-size reuse cache, the trim thresholds and the out-of-memory
+// ladder (the reference's logic is sideaware.cu:1199-1273).  Addresses are made up; nothing is
+// ever dereferenced.
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../l2_torch_alloc_amd/csrc/pool.h"
+
+using namespace sideaware;
+
+namespace {
+
+struct FakeBacking final : Backing {
+    size_t capacity;
+    size_t used = 0;
+    uintptr_t next = 0x7f0000000000ull;          // 2 MiB-aligned, far from real memory
+    std::map<uintptr_t, size_t> live;
+    std::vector<std::string> log;                // "acquire N", "release N", "sync_device", "sync_stream S", "foreign P"
+    int foreign_result = 0;
+
+    explicit FakeBacking(size_t cap) : capacity(cap) {}
+
+    void* acquire(size_t bytes) override {
+        if (used + bytes > capacity) {
+            log.push_back("acquire_failed " + std::to_string(bytes));
+            return nullptr;
+        }
+        uintptr_t p = next;
+        next += (bytes + kRegionAlign - 1) / kRegionAlign * kRegionAlign + kRegionAlign;  // gap: no accidental adjacency
+        used += bytes;
+        live[p] = bytes;
+        log.push_back("acquire " + std::to_string(bytes));
+        return (void*)p;
+    }
+    void release(void* ptr, size_t bytes) override {
+        auto it = live.find((uintptr_t)ptr);
+        if (it == live.end() || it->second != bytes) {
+            log.push_back("bad_release");
+            return;
+        }
+        used -= bytes;
+        live.erase(it);
+        log.push_back("release " + std::to_string(bytes));
+    }
+    void sync_device() override { log.push_back("sync_device"); }
+    void sync_stream(void* s) override { log.push_back("sync_stream " + std::to_string((uintptr_t)s)); }
+    int free_foreign(void* p, void*) override {
+        log.push_back("foreign " + std::to_string((uintptr_t)p));
+        return foreign_result;
+    }
+};
+
+struct Harness {
+    FakeBacking backing;
+    Pool pool;
+    std::string joined;
+    explicit Harness(size_t cap) : backing(cap), pool(&backing) {}
+};
+
+}  // namespace
+
+extern "C" {
+
+void* ph_create(size_t capacity) { return new Harness(capacity); }
+void ph_destroy(void* h) { delete (Harness*)h; }
+
+uintptr_t ph_alloc(void* h, size_t bytes, uintptr_t stream, int always_large) {
+    return (uintptr_t)((Harness*)h)->pool.allocate(bytes, (void*)stream, always_large != 0);
+}
+int ph_free(void* h, uintptr_t ptr, uintptr_t stream) {
+    return ((Harness*)h)->pool.deallocate((void*)ptr, (void*)stream);
+}
+size_t ph_release_unused(void* h) { return ((Harness*)h)->pool.release_unused(); }
+void ph_set_threshold(void* h, size_t t) { ((Harness*)h)->pool.set_large_threshold(t); }
+void ph_set_trim(void* h, size_t a, size_t b) { ((Harness*)h)->pool.set_trim_thresholds(a, b); }
+int ph_owns(void* h, uintptr_t p) { return ((Harness*)h)->pool.owns_live((void*)p) ? 1 : 0; }
+int ph_stats(void* h, uint64_t* out, int cap) {
+    PoolStats s = ((Harness*)h)->pool.stats();
+    int n = cap < kPoolStatsFields ? cap : kPoolStatsFields;
+    std::memcpy(out, &s, n * sizeof(uint64_t));
+    return n;
+}
+size_t ph_backing_used(void* h) { return ((Harness*)h)->backing.used; }
+size_t ph_backing_live_blocks(void* h) { return ((Harness*)h)->backing.live.size(); }
+void ph_set_capacity(void* h, size_t cap) { ((Harness*)h)->backing.capacity = cap; }
+void ph_set_foreign_result(void* h, int r) { ((Harness*)h)->backing.foreign_result = r; }
+const char* ph_log(void* h) {
+    Harness* H = (Harness*)h;
+    H->joined.clear();
+    for (auto& l : H->backing.log) { H->joined += l; H->joined += '\n'; }
+    return H->joined.c_str();
+}
+void ph_clear_log(void* h) { ((Harness*)h)->backing.log.clear(); }
+
+size_t ph_round_large(size_t b) { return Pool::round_large(b); }
+size_t ph_small_class_size(size_t b) { return Pool::small_class_size(b); }
+int ph_small_class_index(size_t b) { return Pool::small_class_index(b); }
+
+}  // extern "C"

@@ -1,0 +1,135 @@
+"""The allocator on a real device, through PyTorch's pluggable-allocator hooks and through the
+direct C entry points (sideaware.cu:1280-1352 are the reference's versions)."""
+import ctypes
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+MiB = 1 << 20
+
+
+def test_torch_tensors_come_from_the_pool(sa):
+    before = sa.sideaware_alloc_stats()
+    big = torch.empty(24 * MiB, dtype=torch.uint8, device="cuda")
+    small = torch.empty(1000, dtype=torch.uint8, device="cuda")
+    after = sa.sideaware_alloc_stats()
+    assert big.data_ptr() % (2 * MiB) == 0
+    assert small.data_ptr() % 512 == 0
+    assert after["large_hits"] + after["large_misses"] == before["large_hits"] + before["large_misses"] + 1
+    assert after["small_hits"] + after["small_carves"] == before["small_hits"] + before["small_carves"] + 1
+    assert after["bytes_live"] >= before["bytes_live"] + 24 * MiB + 1024
+
+
+def test_same_size_blocks_share_the_stripe_phase_and_are_reused(sa):
+    a = torch.empty(40 * MiB, dtype=torch.uint8, device="cuda")
+    b = torch.empty(40 * MiB, dtype=torch.uint8, device="cuda")
+    assert a.data_ptr() % (2 * MiB) == 0 and b.data_ptr() % (2 * MiB) == 0
+    pa = a.data_ptr()
+    del a
+    c = torch.empty(40 * MiB - 100, dtype=torch.uint8, device="cuda")   # rounds to the same 40 MiB
+    assert c.data_ptr() == pa                                             # newest freed block first
+
+
+def test_direct_malloc_free(sa):
+    lib = sa.library()
+    p = ctypes.c_void_p()
+    assert lib.sideaware_malloc(ctypes.byref(p), 3 * MiB + 5) == 0
+    assert p.value and p.value % (2 * MiB) == 0
+    first = p.value
+    assert lib.sideaware_free(p) == 0
+    q = ctypes.c_void_p()
+    assert lib.sideaware_malloc_async(ctypes.byref(q), 4 * MiB, None) == 0
+    assert q.value == first                                               # same rounded size: reused
+    # the memory is real: fill and copy through the kernels
+    r = ctypes.c_void_p()
+    assert lib.sideaware_malloc_async(ctypes.byref(r), 4 * MiB, None) == 0
+    host = torch.arange(MiB, dtype=torch.int32)
+    dev = host.cuda()
+    lib.sideaware_memcpy(q, dev.data_ptr(), 4 * MiB, 0, None)
+    lib.sideaware_memcpy(r, q, 4 * MiB, 0, None)
+    back = torch.zeros_like(dev)
+    lib.sideaware_memcpy(back.data_ptr(), r, 4 * MiB, 0, None)
+    torch.cuda.synchronize()
+    assert torch.equal(back.cpu(), host)
+    assert lib.sideaware_free_async(q, None) == 0
+    assert lib.sideaware_free_async(r, None) == 0
+    assert lib.sideaware_free_async(None, None) == 0
+
+
+def test_release_unused_gives_memory_back(sa):
+    lib = sa.library()
+    x = torch.empty(64 * MiB, dtype=torch.uint8, device="cuda")
+    del x
+    torch.cuda.synchronize()
+    cached = sa.sideaware_alloc_stats()["bytes_cached_large"]
+    assert cached >= 64 * MiB
+    freed = lib.sideaware_release_unused()
+    assert freed >= cached
+    assert sa.sideaware_alloc_stats()["bytes_cached_large"] == 0
+
+
+def test_out_of_memory_is_a_torch_exception_not_a_crash(sa):
+    total = torch.cuda.get_device_properties(0).total_memory
+    with pytest.raises(torch.OutOfMemoryError):
+        torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
+    assert sa.sideaware_alloc_stats()["failures"] >= 1
+    sa.library().sideaware_clear_error()
+    # and the pool still serves requests afterwards
+    y = torch.ones(10 * MiB, dtype=torch.uint8, device="cuda")
+    assert int(y.sum()) == 10 * MiB
+
+
+def test_threshold_and_trim_settings_apply(sa):
+    lib = sa.library()
+    lib.sideaware_free_mapped_thresholds(32 * MiB, 0)
+    try:
+        blocks = [torch.empty((10 + 2 * i) * MiB, dtype=torch.uint8, device="cuda") for i in range(6)]
+        del blocks
+        assert sa.sideaware_alloc_stats()["bytes_cached_large"] >= 90 * MiB
+        trims = sa.sideaware_alloc_stats()["trims"]
+        z = torch.empty(50 * MiB, dtype=torch.uint8, device="cuda")     # a miss, cache over budget
+        st = sa.sideaware_alloc_stats()
+        assert st["trims"] == trims + 1 and st["bytes_cached_large"] == 0
+        del z
+    finally:
+        lib.sideaware_free_mapped_thresholds(16 << 30, 2 << 30)
+    lib.sideaware_alloc_threshold(1 * MiB)
+    try:
+        t = torch.empty(MiB, dtype=torch.uint8, device="cuda")
+        assert t.data_ptr() % (2 * MiB) == 0
+    finally:
+        lib.sideaware_alloc_threshold(8 * MiB)
+
+
+def test_churn_contents_survive(sa):
+    # tensors of random sizes filled with a tag; whatever the pool recycles, live data must stay put
+    rng = random.Random(7)
+    live = []
+    for step in range(400):
+        if live and rng.random() < 0.5:
+            t, tag = live.pop(rng.randrange(len(live)))
+            assert int(t[0]) == tag and int(t[-1]) == tag
+        else:
+            n = int(4096 * 2 ** (rng.random() * 14)) // 4
+            tag = step
+            t = torch.full((n,), tag, dtype=torch.int32, device="cuda")
+            live.append((t, tag))
+    for t, tag in live:
+        assert bool((t == tag).all())
+
+
+def test_memcpy_under_torch_compile(sa):
+    # the custom op traces with fullgraph=True (test.py:175-184)
+    @torch.compile(fullgraph=True)
+    def compiled_copy(dst, src):
+        torch.ops.sideaware.memcpy(dst, src)
+        return dst
+
+    src = torch.ones((8, 8), dtype=torch.float32, device="cuda") * 2.0
+    dst = torch.zeros((8, 8), dtype=torch.float32, device="cuda")
+    out = compiled_copy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(out, src) and torch.equal(dst, src)

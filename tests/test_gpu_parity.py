@@ -1,0 +1,390 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+memcpy, fill and the mixed-width op are bit-exact.  fp32 RoPE is held to 1e-6 relative
+(|got - want| <= 1e-6 * max(|want|, tiny)), and is expected to be bit-identical because neither
+side fuses multiply and add; bf16 RoPE and scale+bias are held to 1 bf16 ulp, again expected
+exact.  Full-size cases run at the shapes of the benchmark workloads; where the oracle would be
+slow, size-independent properties take over (backward(forward(x)) == x, equality of two runs).
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+MiB = 1 << 20
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    """Host copy of a tensor's raw bytes as an unsigned integer array (NaN-safe comparisons)."""
+    t = t.detach().contiguous().cpu()
+    view = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
+    return t.view(view).numpy().view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[t.element_size()])
+
+
+def bf16_tensor(bits_u16: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(bits_u16.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def assert_no_library_error(sa):
+    assert sa.sideaware_last_error() == "", sa.sideaware_last_error()
+
+
+# --------------------------------------------------------------------------------------- start-up
+
+def test_metadata(sa):
+    info = sa.sideaware_info()
+    lib = sa.library()
+    print("sideaware metadata:", info, "xcds:", lib.sideaware_num_xcds(),
+          "dealing verified:", lib.sideaware_xcd_dealing_verified())
+    assert info["num_sms"] == torch.cuda.get_device_properties(0).multi_processor_count
+    assert lib.sideaware_num_xcds() >= 1
+    assert info["num_sms"] % lib.sideaware_num_xcds() == 0
+    assert info["min"] >= 1 and info["hash"] & (1 << 21)
+    table = sa.sideaware_torch_side_index().cpu().numpy()
+    assert table.shape == (info["num_sms"],)
+    xcd = table & 7
+    counts = np.bincount(xcd, minlength=lib.sideaware_num_xcds())
+    assert counts.sum() == info["num_sms"] and counts[0] == info["side0"]
+    # ranks within each XCD count up from zero without gaps
+    for x in range(lib.sideaware_num_xcds()):
+        ranks = np.sort(table[xcd == x] >> 3)
+        assert np.array_equal(ranks, np.arange(len(ranks)) & 0x1f)
+    # the host copy the library returns a pointer to holds the same bytes
+    host = (ctypes.c_ubyte * info["num_sms"]).from_address(sa.sideaware_cpu_side_index())
+    assert np.array_equal(np.frombuffer(host, dtype=np.uint8), table)
+
+
+# --------------------------------------------------------------------------------------- memcpy
+
+@pytest.mark.parametrize("nbytes", [16, 256, 4096, 12432, 16384, 16400, 65536 + 4080, MiB, 8 * MiB,
+                                    8 * MiB + 48, 64 * MiB, 256 * MiB])
+def test_memcpy_bit_exact(sa, nbytes):
+    g = torch.Generator().manual_seed(nbytes)
+    src_host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g)
+    src = src_host.cuda()
+    dst = torch.full((nbytes + 512,), 0xA5, dtype=torch.uint8, device="cuda")   # 256 guard bytes each side
+    inner = dst[256:256 + nbytes]
+    torch.ops.sideaware.memcpy(inner, src)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    out = dst.cpu()
+    assert torch.equal(out[256:256 + nbytes], src_host)
+    assert bool((out[:256] == 0xA5).all()) and bool((out[256 + nbytes:] == 0xA5).all())
+    assert np.array_equal(O.memcpy(src_host.numpy()), out[256:256 + nbytes].numpy())
+
+
+def test_memcpy_aligned_regions_take_the_fast_variant(sa):
+    # two fresh 256 MiB tensors come straight from the large pool: 2 MiB-aligned, same stripe phase
+    n = 256 * MiB
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    assert src.data_ptr() % (2 * MiB) == 0 and dst.data_ptr() % (2 * MiB) == 0
+    torch.ops.sideaware.memcpy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    assert_no_library_error(sa)
+
+
+@pytest.mark.parametrize("dtype,shape,start", [
+    (torch.float32, (4, 777), 0),            # 12,432 bytes: all tail (test.py:310)
+    (torch.int16, (1000, 1000), 0),          # test.py:314
+    (torch.float64, (1000, 1000), 0),        # test.py:315
+    (torch.float32, (10000, 1000), 0),       # ~40 MB (test.py:316)
+    (torch.float32, (10000, 1000), 3),       # a slice: base 12,000 bytes into the region
+    (torch.bfloat16, (3, 5, 7, 64), 1),
+])
+def test_memcpy_shapes_and_dtypes_vs_copy_(sa, dtype, shape, start):
+    n = int(np.prod(shape))
+    src = torch.arange(n, device="cuda").to(dtype).reshape(shape)
+    dst_ours = torch.zeros_like(src)
+    dst_torch = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(dst_ours[start:], src[start:])
+    dst_torch[start:].copy_(src[start:])
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(dst_ours), bits(dst_torch))
+    assert_no_library_error(sa)
+
+
+def test_memcpy_nan_payloads_survive(sa):
+    pattern = torch.tensor([0x7FC00001, 0xFFC12345 - (1 << 32), 0x7F800001, 0], dtype=torch.int32).repeat(1024)
+    src = pattern.cuda().view(torch.float32)
+    dst = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(dst, src)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(dst), bits(src))
+
+
+def test_memcpy_needs_64_bit_indices(sa):
+    # 2 GiB + 64 KiB + 16 B: past the 32-bit path of the launcher (sideaware.cu:1387) and with a tail
+    n = (2 << 30) + 65536 + 16
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    src.view(torch.int64)[: n // 8] = torch.arange(n // 8, device="cuda", dtype=torch.int64) * 0x9E3779B97F4A7C15
+    dst = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    assert_no_library_error(sa)
+
+
+def test_memcpy_6gb_like_the_reference_script(sa):
+    # (100000, 15000) fp32 = 6 GB (test.py:311)
+    src = torch.arange(100000 * 15000, dtype=torch.float32, device="cuda").reshape(100000, 15000)
+    dst = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
+
+
+def test_memcpy_on_a_side_stream(sa):
+    n = 32 * MiB
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        torch.ops.sideaware.memcpy(dst, src)
+    stream.synchronize()
+    assert torch.equal(dst, src)
+
+
+def test_launch_knobs_do_not_change_results(sa):
+    n = 24 * MiB + 4096 + 32
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    lib = sa.library()
+    for groups, per_xcd in [(1, 0), (2, 1), (3, 5), (8, 0), (16, 31)]:
+        dst = torch.zeros_like(src)
+        lib.sideaware_elementwise(0, n, dst.data_ptr(), 0, 0, 0, src.data_ptr(), 0, 0, 0, 0, 0,
+                                  groups, per_xcd, 0, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src), (groups, per_xcd)
+    assert_no_library_error(sa)
+
+
+def test_misuse_is_reported_not_fatal(sa):
+    lib = sa.library()
+    x = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    y = torch.ones(4096, dtype=torch.uint8, device="cuda")
+    lib.sideaware_clear_error()
+    lib.sideaware_memcpy(x.data_ptr() + 8, y.data_ptr(), 1024, 0, None)       # 8-byte aligned only
+    assert "multiples of 16" in sa.sideaware_last_error()
+    lib.sideaware_clear_error()
+    lib.sideaware_memcpy(x.data_ptr(), y.data_ptr(), 1000, 0, None)           # length not a multiple of 16
+    assert "multiples of 16" in sa.sideaware_last_error()
+    lib.sideaware_clear_error()
+    lib.sideaware_one_to_one(9999, 1024, x.data_ptr(), y.data_ptr(), 0, None)
+    assert "never created" in sa.sideaware_last_error()
+    bad = lib.sideaware_create_kernel(b"typedef int o0; this does not compile")
+    lib.sideaware_clear_error()
+    lib.sideaware_one_to_one(bad, 1024, x.data_ptr(), y.data_ptr(), 0, None)
+    assert "failed to compile" in sa.sideaware_last_error()
+    torch.cuda.synchronize()
+    assert int(x.sum()) == 0                                                   # nothing ran
+    lib.sideaware_clear_error()
+
+
+# --------------------------------------------------------------------------------------- custom ops
+
+MIXED_HEADER = b"""
+#include <cuda_fp16.h>
+#include <cuda_bf16.h>
+typedef float o0;
+typedef half o1;
+typedef __nv_bfloat16 i0;
+typedef float i1;
+struct unused {};
+typedef unused o2, o3, i2, i3;
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = (o0)((float)in0 + (float)in1);
+    out1 = (o1)((float)in1 * 10.0f);
+}
+constexpr bool reverse_order = true;
+constexpr bool input_evict[4] = {1,1,1,1};
+"""
+
+
+@pytest.mark.parametrize("n", [64, 1024 * 1024 + 64])
+def test_two_in_two_out_mixed_widths(sa, n):
+    # the reference's run-time-compile check (test.py:218-230): small integers, exact in bf16/fp16
+    in0 = (torch.arange(n, device="cuda", dtype=torch.float32) % 64).to(torch.bfloat16)
+    in1 = torch.ones(n, device="cuda", dtype=torch.float32) * 2
+    out0 = torch.zeros(n, device="cuda", dtype=torch.float32)
+    out1 = torch.zeros(n, device="cuda", dtype=torch.float16)
+    kid = sa.sideaware_create_kernel(MIXED_HEADER)
+    torch.ops.sideaware.elementwise(kid, out0, out1, None, None, in0, in1, None, None, None, 0, 0, 0)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert torch.equal(out0, in0.float() + in1)
+    assert torch.equal(out1, (in1 * 10.0).half())
+
+
+def test_output_only_fill(sa):
+    from l2_torch_alloc_amd import ops
+    out = torch.zeros(3 * MiB // 4 + 4, dtype=torch.int32, device="cuda")
+    ops.fill_int32(out, 0x5EEDBEEF)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert bool((out == 0x5EEDBEEF).all())
+
+
+def test_scale_bias_bf16_vs_oracle_and_golden(sa):
+    from l2_torch_alloc_amd import ops
+    g = np.load(os.path.join(GOLDEN, "scale_bias_bf16.npz"))
+    x = bf16_tensor(g["x"]).cuda()
+    sb = torch.tensor([float(g["scale"]), float(g["bias"])], dtype=torch.float32, device="cuda")
+    y = ops.scale_bias_bf16(x, sb)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), g["y"])
+    # a larger seeded case against the oracle directly, other constants, same compiled kernel
+    gen = torch.Generator().manual_seed(5)
+    xh = torch.randn(5 * MiB + 8, generator=gen).to(torch.bfloat16)
+    sb2 = torch.tensor([1.7, -0.3], dtype=torch.float32, device="cuda")
+    y2 = ops.scale_bias_bf16(xh.cuda(), sb2)
+    torch.cuda.synchronize()
+    want = O.scale_bias_bf16(bits(xh), float(np.float32(1.7)), float(np.float32(-0.3)))
+    assert O.bf16_ulp_distance(bits(y2), want).max() <= 1
+    assert np.array_equal(bits(y2), want)
+    assert_no_library_error(sa)
+
+
+# --------------------------------------------------------------------------------------- RoPE
+
+def rel_err(got: np.ndarray, want: np.ndarray) -> float:
+    return float(np.max(np.abs(got.astype(np.float64) - want) / np.maximum(np.abs(want), 1e-30)))
+
+
+FP32_REL_TOL = 1e-6
+
+
+@pytest.mark.parametrize("name", ["rope_fp32_qkv_tiny", "rope_fp32_qkv_gqa", "rope_fp32_qkv_scaled",
+                                  "rope_fp32_heads_gpt2"])
+def test_rope_fp32_golden(sa, name):
+    from l2_torch_alloc_amd import ops
+    g = np.load(os.path.join(GOLDEN, name + ".npz"))
+    B, T, Nq, Nkv, HS = (int(v) for v in g["shape"])
+    x = torch.from_numpy(g["x"]).cuda()
+    freqs = torch.from_numpy(g["freqs"]).cuda()
+    if "qkv" in name:
+        y = ops.rope_forward_qkv(x.clone(), freqs, Nq, Nkv)
+        dx = ops.rope_backward_qkv(y.clone(), freqs, Nq, Nkv)
+    else:
+        y = ops.rope_forward_heads(x.clone(), freqs)
+        dx = ops.rope_backward_heads(y.clone(), freqs)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(y), g["y"].view(np.uint32))
+    assert np.array_equal(bits(dx), g["dx"].view(np.uint32))
+
+
+def test_rope_bf16_golden(sa):
+    from l2_torch_alloc_amd import ops
+    g = np.load(os.path.join(GOLDEN, "rope_bf16_heads_llama3.npz"))
+    x = bf16_tensor(g["x"]).cuda()
+    y = ops.rope_forward_heads(x, torch.from_numpy(g["freqs"]).cuda())
+    torch.cuda.synchronize()
+    assert O.bf16_ulp_distance(bits(y), g["y"]).max() <= 1
+    assert np.array_equal(bits(y), g["y"])
+
+
+def test_rope_fp32_gpt2_shape_vs_oracle(sa):
+    # (B=4, T=1024, NH=12, HS=64) fp32, theta 1e4: in place and out of place
+    from l2_torch_alloc_amd import ops
+    B, T, NH, HS = 4, 1024, 12, 64
+    gen = torch.Generator().manual_seed(1)
+    xh = torch.randn(B, T, NH, HS, generator=gen)
+    freqs_h = O.freqs_cis(HS, T, 10000.0)
+    want = O.rope_forward_heads_f32(xh.numpy(), freqs_h)
+    freqs = torch.from_numpy(freqs_h).cuda()
+    x = xh.cuda()
+    out = torch.empty_like(x)
+    ops.rope_forward_heads(x, freqs, out=out)
+    inplace = ops.rope_forward_heads(x.clone(), freqs)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    got = out.cpu().numpy()
+    assert rel_err(got, want) <= FP32_REL_TOL
+    assert O.validate_f32(got, want, 1e-5) == 0           # the reference harness's own rule
+    assert np.array_equal(bits(out), want.view(np.uint32)), "expected bit-identical fp32"
+    assert torch.equal(inplace, out)
+    assert torch.equal(x.cpu(), xh)                       # out-of-place left the input alone
+
+
+def test_rope_fp32_packed_qkv_reference_shape_vs_oracle(sa):
+    # the reference benchmark's own tensor: (8, 1024, 3*32, 128) fp32, theta 1e4 with Llama-3.1
+    # scaling (example_llmc_rope.cu:249-260); value heads must come through untouched
+    from l2_torch_alloc_amd import ops
+    B, T, NH, HS = 8, 1024, 32, 128
+    gen = torch.Generator().manual_seed(8)
+    xh = torch.randn(B, T, 3 * NH, HS, generator=gen)
+    freqs_h = O.freqs_cis(HS, T, 10000.0, use_scaled=True)
+    want = O.rope_forward_qkv_f32(xh.numpy(), freqs_h, NH, NH)
+    x = xh.cuda()
+    ops.rope_forward_qkv(x, torch.from_numpy(freqs_h).cuda(), NH, NH)
+    torch.cuda.synchronize()
+    got = x.cpu().numpy()
+    assert rel_err(got, want) <= FP32_REL_TOL
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(got[:, :, 2 * NH:].view(np.uint32), xh.numpy()[:, :, 2 * NH:].view(np.uint32))
+    # backward brings it back (conjugate rotation), to rounding
+    ops.rope_backward_qkv(x, torch.from_numpy(freqs_h).cuda(), NH, NH)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(x.cpu().numpy(), xh.numpy(), atol=2e-6, rtol=2e-6)
+    want_back = O.rope_backward_qkv_f32(want, freqs_h, NH, NH)
+    assert np.array_equal(bits(x), want_back.view(np.uint32))
+
+
+def test_rope_out_of_place_qkv_carries_value_heads(sa):
+    from l2_torch_alloc_amd import ops
+    B, T, Nq, Nkv, HS = 2, 16, 4, 2, 64
+    xh = torch.randn(B, T, Nq + 2 * Nkv, HS, generator=torch.Generator().manual_seed(3))
+    freqs_h = O.freqs_cis(HS, T, 500000.0)
+    out = torch.full_like(xh, float("nan")).cuda()
+    ops.rope_forward_qkv(xh.cuda(), torch.from_numpy(freqs_h).cuda(), Nq, Nkv, out=out)
+    torch.cuda.synchronize()
+    want = O.rope_forward_qkv_f32(xh.numpy(), freqs_h, Nq, Nkv)
+    assert np.array_equal(bits(out), want.view(np.uint32))
+
+
+def test_rope_bf16_llama3_full_size_vs_oracle(sa):
+    # q (8, 4096, 32, 128) and k (8, 4096, 8, 128) bf16 in place, theta 5e5: the benchmark workload
+    from l2_torch_alloc_amd import ops
+    B, T, HS = 8, 4096, 128
+    freqs_h = O.freqs_cis(HS, T, 500000.0)
+    freqs = torch.from_numpy(freqs_h).cuda()
+    gen = torch.Generator().manual_seed(2)
+    for heads in (32, 8):
+        xh = torch.randn(B, T, heads, HS, generator=gen).to(torch.bfloat16)
+        x = xh.cuda()
+        assert x.data_ptr() % (2 * MiB) == 0
+        ops.rope_forward_heads(x, freqs)
+        torch.cuda.synchronize()
+        assert_no_library_error(sa)
+        want = O.rope_forward_heads_bf16(bits(xh), freqs_h)
+        got = bits(x)
+        dist = O.bf16_ulp_distance(got, want)
+        assert dist.max() <= 1, "more than 1 bf16 ulp from the fp32 oracle"
+        assert np.array_equal(got, want), "expected bit-identical bf16 (%d differ)" % int((dist > 0).sum())
+        del x, xh, want, got, dist
+
+
+def test_rope_bf16_packed_gqa_vs_oracle(sa):
+    # packed QKV with grouped heads in bf16: oracle = rotate the q|k slice as heads, keep v bits
+    from l2_torch_alloc_amd import ops
+    B, T, Nq, Nkv, HS = 2, 512, 32, 8, 128
+    xh = torch.randn(B, T, Nq + 2 * Nkv, HS, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16)
+    freqs_h = O.freqs_cis(HS, T, 500000.0)
+    x = xh.cuda()
+    ops.rope_forward_qkv(x, torch.from_numpy(freqs_h).cuda(), Nq, Nkv)
+    torch.cuda.synchronize()
+    xb = bits(xh)
+    want = xb.copy()
+    want[:, :, :Nq + Nkv] = O.rope_forward_heads_bf16(np.ascontiguousarray(xb[:, :, :Nq + Nkv]), freqs_h)
+    assert np.array_equal(bits(x), want)

@@ -68,21 +68,23 @@ def lib():
     return L
 
 
-def build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse):
+def build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse, header=None):
     assert lib.sideaware_tune(b"stripe_bytes", stripe) == 0
     config = lib.sideaware_config_block(variant).decode()
     template = lib.sideaware_kernel_source().decode()
-    header = (INCREMENT_HEADER if case == "INCREMENT" else MIXED_HEADER) % {
-        "reverse": "true" if reverse else "false",
-        "unrolled": "" if unrolled is None else "#define UNROLLED %d" % unrolled,
-    }
+    if header is None:
+        header = (INCREMENT_HEADER if case == "INCREMENT" else MIXED_HEADER) % {
+            "reverse": "true" if reverse else "false",
+            "unrolled": "" if unrolled is None else "#define UNROLLED %d" % unrolled,
+        }
     tu = "\n".join([
         '#include "%s"' % os.path.join(NATIVE, "kernel_cpu_prelude.h"),
         config, header, template,
         "#define SA_CASE_%s 1" % case,
         '#include "%s"' % os.path.join(NATIVE, "kernel_cpu_driver.h"),
     ])
-    src = tmp_path / ("tu_%s_v%d_u%s_s%d_r%d.cpp" % (case, variant, unrolled, stripe, reverse))
+    src = tmp_path / ("tu_%s_v%d_u%s_s%d_r%d_%x.cpp" % (case, variant, unrolled, stripe, reverse,
+                                                        hash(header) & 0xffffff))
     exe = str(src)[:-4]
     src.write_text(tu)
     cmd = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
@@ -131,6 +133,42 @@ def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, stripe, reverse
     cases = cases_for(variant, unrolled, rng)
     if case == "MIXED":
         cases = [(g, n, off - off % 64) for (g, n, off) in cases]   # halves of the offset stay 16 B-aligned
+    text = "".join("%d %d %d\n" % c for c in cases)
+    proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
+                          env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
+    assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
+    assert "cases=%d failed=0" % len(cases) in proc.stdout
+
+
+ROPE_SHAPES = [
+    # T, n_q, n_kv, head_dim, dtype, layout, backward-free forward only; variant
+    (8, 3, 3, 8, "fp32", "qkv", 0),
+    (16, 12, 12, 64, "fp32", "qkv", 1),
+    (5, 4, 1, 16, "fp32", "qkv", 1),          # GQA head counts, T not a power of two
+    (8, 32, 0, 128, "bf16", "heads", 0),
+    (6, 8, 0, 128, "bf16", "heads", 1),
+    (4, 4, 2, 32, "bf16", "qkv", 1),
+]
+
+
+@pytest.mark.parametrize("T,n_q,n_kv,head_dim,dtype,layout,variant", ROPE_SHAPES)
+def test_rope_headers_on_cpu(lib, tmp_path, T, n_q, n_kv, head_dim, dtype, layout, variant):
+    if not os.path.exists(CLANG):
+        pytest.skip("ROCm clang++ not found")
+    from l2_torch_alloc_amd import headers
+    header = headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout).decode()
+    exe = build_driver(lib, tmp_path, "ROPE", variant, None, 16384, False, header=header)
+    heads = n_q + 2 * n_kv if layout == "qkv" else n_q
+    pair_bytes = 8 if dtype == "fp32" else 4
+    vecs_per_token = heads * (head_dim // 2) * pair_bytes // 16
+    rng = random.Random(T * 131 + heads)
+    cases = []
+    for tokens in (1, T - 1, T, T + 1, 3 * T, 7 * T + 2):
+        nv = tokens * vecs_per_token
+        for grid in rng.sample([8, 16, 56, 2048], 2):
+            for off in ([0] if variant == 0 else [0, 16, 4096 + 32]):
+                cases.append((grid, nv, off))
+    cases.append((8, 3 * vecs_per_token + 1, 0))       # length that is not a whole number of tokens
     text = "".join("%d %d %d\n" % c for c in cases)
     proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
                           env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))

@@ -1,0 +1,314 @@
+"""Allocator policy on the CPU: the real ``Pool`` (l2_torch_alloc_amd/csrc/pool.cpp) over a fake
+backing store.
+
+What the reference promises and this pool must keep (sideaware.cu:1199-1273, 1320-1352):
+exact-size LIFO reuse of large blocks, 2 MiB rounding and alignment, blocks stay cached on free,
+cached bytes above the start threshold are trimmed to the end threshold on a miss, a four-step
+ladder before giving up with a null pointer, free(null) is a no-op, unknown pointers are
+forwarded to the runtime.  Added here: pooled size classes for small requests, double-free
+detection, stream hand-over syncs.
+"""
+import ctypes
+import os
+import random
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SRC = os.path.join(HERE, "native", "pool_harness.cpp")
+POOL = os.path.join(ROOT, "l2_torch_alloc_amd", "csrc", "pool.cpp")
+LIB = os.path.join(HERE, "native", "libpool_harness.so")
+
+MiB = 1 << 20
+GiB = 1 << 30
+FIELDS = ("large_hits", "large_misses", "small_hits", "small_carves", "slabs_acquired", "backing_acquires",
+          "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
+          "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
+          "peak_reserved")
+
+
+def build_harness():
+    newest = max(os.path.getmtime(p) for p in (SRC, POOL, POOL[:-4] + ".h"))
+    if not os.path.exists(LIB) or os.path.getmtime(LIB) < newest:
+        subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fPIC", "-shared", "-Wall", SRC, POOL, "-o", LIB],
+                       check=True)
+    return LIB
+
+
+@pytest.fixture(scope="module")
+def ph():
+    L = ctypes.CDLL(build_harness())
+    u, sz, vp = ctypes.c_uint64, ctypes.c_size_t, ctypes.c_void_p
+    L.ph_create.restype, L.ph_create.argtypes = vp, [sz]
+    L.ph_destroy.argtypes = [vp]
+    L.ph_alloc.restype, L.ph_alloc.argtypes = u, [vp, sz, u, ctypes.c_int]
+    L.ph_free.restype, L.ph_free.argtypes = ctypes.c_int, [vp, u, u]
+    L.ph_release_unused.restype, L.ph_release_unused.argtypes = sz, [vp]
+    L.ph_set_threshold.argtypes = [vp, sz]
+    L.ph_set_trim.argtypes = [vp, sz, sz]
+    L.ph_owns.restype, L.ph_owns.argtypes = ctypes.c_int, [vp, u]
+    L.ph_stats.restype, L.ph_stats.argtypes = ctypes.c_int, [vp, ctypes.POINTER(u), ctypes.c_int]
+    L.ph_backing_used.restype, L.ph_backing_used.argtypes = sz, [vp]
+    L.ph_backing_live_blocks.restype, L.ph_backing_live_blocks.argtypes = sz, [vp]
+    L.ph_set_capacity.argtypes = [vp, sz]
+    L.ph_set_foreign_result.argtypes = [vp, ctypes.c_int]
+    L.ph_log.restype, L.ph_log.argtypes = ctypes.c_char_p, [vp]
+    L.ph_clear_log.argtypes = [vp]
+    L.ph_round_large.restype, L.ph_round_large.argtypes = sz, [sz]
+    L.ph_small_class_size.restype, L.ph_small_class_size.argtypes = sz, [sz]
+    L.ph_small_class_index.restype, L.ph_small_class_index.argtypes = ctypes.c_int, [sz]
+    return L
+
+
+class P:
+    def __init__(self, L, capacity=64 * GiB):
+        self.L, self.h = L, L.ph_create(capacity)
+
+    def close(self):
+        self.L.ph_destroy(self.h)
+
+    def alloc(self, n, stream=0, large=False):
+        return self.L.ph_alloc(self.h, n, stream, int(large))
+
+    def free(self, p, stream=0):
+        return self.L.ph_free(self.h, p, stream)
+
+    def stats(self):
+        buf = (ctypes.c_uint64 * len(FIELDS))()
+        n = self.L.ph_stats(self.h, buf, len(FIELDS))
+        assert n == len(FIELDS)
+        return dict(zip(FIELDS, buf))
+
+    def log(self):
+        return self.L.ph_log(self.h).decode().splitlines()
+
+    def clear_log(self):
+        self.L.ph_clear_log(self.h)
+
+
+@pytest.fixture
+def pool(ph):
+    p = P(ph)
+    yield p
+    p.close()
+
+
+# ------------------------------------------------------------------------------ rounding rules
+
+def test_round_large(ph):
+    assert ph.ph_round_large(1) == 2 * MiB
+    assert ph.ph_round_large(2 * MiB) == 2 * MiB
+    assert ph.ph_round_large(2 * MiB + 1) == 4 * MiB
+    assert ph.ph_round_large(512 * MiB) == 512 * MiB
+
+
+def test_small_classes_monotone_tight_and_aligned(ph):
+    prev_size, prev_idx = 0, -1
+    for n in list(range(1, 70000, 37)) + [2 ** k + d for k in range(9, 33) for d in (-1, 0, 1)]:
+        c = ph.ph_small_class_size(n)
+        assert c >= n and c % 512 == 0
+        assert c - n <= max(511, n // 8 + 1), (n, c)      # at most 12.5 % slack above 4 KiB
+        assert ph.ph_small_class_size(c) == c              # a class size is its own class
+        assert ph.ph_small_class_index(n) == ph.ph_small_class_index(c)
+    sizes = sorted({ph.ph_small_class_size(n) for n in range(1, 1 << 20, 101)})
+    idx = [ph.ph_small_class_index(s) for s in sizes]
+    assert idx == sorted(idx) and len(set(idx)) == len(idx)   # distinct sizes, distinct slots, same order
+
+
+# ------------------------------------------------------------------------------ large path
+
+def test_large_is_2mib_aligned_rounded_and_reused_lifo(pool):
+    a = pool.alloc(9 * MiB)
+    b = pool.alloc(9 * MiB + 5)          # rounds to the same 10 MiB
+    assert a % (2 * MiB) == 0 and b % (2 * MiB) == 0 and a != b
+    assert pool.stats()["bytes_live"] == 20 * MiB
+    pool.free(a)
+    pool.free(b)
+    s = pool.stats()
+    assert s["bytes_live"] == 0 and s["bytes_cached_large"] == 20 * MiB
+    assert s["backing_releases"] == 0                        # freed blocks stay cached
+    assert pool.alloc(10 * MiB) == b                         # newest first
+    assert pool.alloc(9 * MiB + 1) == a
+    assert pool.stats()["large_hits"] == 2
+    c = pool.alloc(12 * MiB)                                 # another size: no reuse
+    assert c not in (a, b) and pool.stats()["large_misses"] == 3
+
+
+def test_direct_entry_points_are_always_large(pool):
+    p = pool.alloc(100, large=True)
+    assert p % (2 * MiB) == 0 and pool.stats()["bytes_live"] == 2 * MiB
+
+
+def test_threshold_moves_the_boundary(pool):
+    pool.L.ph_set_threshold(pool.h, 1 * MiB)
+    p = pool.alloc(1 * MiB)
+    assert p % (2 * MiB) == 0 and pool.stats()["large_misses"] == 1
+    q = pool.alloc(1 * MiB - 1)
+    assert pool.stats()["small_carves"] == 1 and q != p
+
+
+def test_stream_handover_syncs_the_old_stream(pool):
+    a = pool.alloc(16 * MiB, stream=11)
+    pool.free(a, stream=11)
+    pool.clear_log()
+    assert pool.alloc(16 * MiB, stream=11) == a
+    assert pool.log() == []                                  # same stream: reuse is stream-ordered
+    pool.free(a, stream=11)
+    assert pool.alloc(16 * MiB, stream=22) == a
+    assert pool.log() == ["sync_stream 11"]
+    s = pool.alloc(4096, stream=5)
+    pool.free(s, stream=5)
+    pool.clear_log()
+    assert pool.alloc(4096, stream=6) == s
+    assert pool.log() == ["sync_stream 5"]
+
+
+def test_trim_thresholds(pool):
+    pool.L.ph_set_trim(pool.h, 64 * MiB, 16 * MiB)
+    blocks = [pool.alloc((8 + 2 * i) * MiB) for i in range(8)]     # 8..22 MiB, 120 MiB total
+    for b in blocks:
+        pool.free(b)
+    assert pool.stats()["bytes_cached_large"] == 120 * MiB
+    pool.clear_log()
+    p = pool.alloc(100 * MiB)                                      # a miss with the cache over budget
+    assert p
+    s = pool.stats()
+    assert s["trims"] == 1 and s["bytes_cached_large"] <= 16 * MiB
+    log = pool.log()
+    assert log[0] == "sync_device"                                 # drained before memory goes back
+    assert log[-1] == "acquire %d" % (100 * MiB)
+    # a hit never trims, whatever the cache holds
+    pool.free(p)
+    before = pool.stats()["backing_releases"]
+    assert pool.alloc(100 * MiB) == p
+    assert pool.stats()["backing_releases"] == before
+
+
+def test_oom_ladder_and_null(ph):
+    pool = P(ph, capacity=64 * MiB)
+    try:
+        a = pool.alloc(20 * MiB)
+        b = pool.alloc(20 * MiB)
+        small = pool.alloc(4096)                 # a 2 MiB slab
+        pool.free(a)
+        pool.free(b)
+        pool.free(small)
+        # 40 MiB cached + 2 MiB slab held; 44 MiB only fits once the caches are given back
+        pool.clear_log()
+        c = pool.alloc(44 * MiB)
+        assert c
+        log = pool.log()
+        assert log[0] == "acquire_failed %d" % (44 * MiB)          # step 2
+        assert "release %d" % (20 * MiB) in log                    # step 3 gives the cache back
+        s = pool.stats()
+        assert s["ladder_retries"] >= 1 and s["failures"] == 0
+        # nothing can make 128 MiB fit: every step is walked, then null
+        pool.clear_log()
+        assert pool.alloc(128 * MiB) == 0
+        s = pool.stats()
+        assert s["failures"] == 1
+        assert pool.log().count("acquire_failed %d" % (128 * MiB)) == 3
+        # the pool is still usable afterwards
+        pool.free(c)
+        assert pool.alloc(44 * MiB) == c
+    finally:
+        pool.close()
+
+
+def test_release_unused_returns_everything_cached(pool):
+    a = pool.alloc(32 * MiB)
+    smalls = [pool.alloc(1000) for _ in range(10)]
+    keep = pool.alloc(3000)
+    pool.free(a)
+    for s in smalls:
+        pool.free(s)
+    released = pool.L.ph_release_unused(pool.h)
+    assert released == 32 * MiB + 2 * MiB             # the large block and the now-empty 1 KiB-class slab
+    st = pool.stats()
+    assert st["bytes_cached_large"] == 0
+    assert pool.L.ph_backing_live_blocks(pool.h) == 1  # only the slab that holds `keep`
+    assert pool.L.ph_owns(pool.h, keep)
+    # and the classes still work after their slabs were taken away
+    again = pool.alloc(1000)
+    assert again and pool.L.ph_owns(pool.h, again)
+
+
+# ------------------------------------------------------------------------------ small path
+
+def test_small_blocks_are_pooled_and_512_aligned(pool):
+    ptrs = [pool.alloc(n) for n in (1, 511, 512, 513, 4096, 4097, 100000, 7 * MiB)]
+    assert all(p and p % 512 == 0 for p in ptrs)
+    assert len(set(ptrs)) == len(ptrs)
+    s = pool.stats()
+    assert s["small_carves"] == len(ptrs) and s["large_misses"] == 0
+    pool.free(ptrs[2])
+    assert pool.alloc(400) == ptrs[2]                 # same class (512 B) comes straight back
+    assert pool.stats()["small_hits"] == 1
+
+
+def test_many_small_allocs_reach_the_backing_rarely(pool):
+    ptrs = [pool.alloc(4096) for _ in range(1000)]
+    assert pool.stats()["slabs_acquired"] <= 2        # 64 KiB-per-16 rule => 2 MiB slabs of 512 blocks
+    for p in ptrs:
+        pool.free(p)
+    for _ in range(1000):
+        assert pool.alloc(4096) in ptrs
+    assert pool.stats()["slabs_acquired"] <= 2
+
+
+def test_double_free_and_interior_pointer_are_refused(pool):
+    p = pool.alloc(2048)
+    assert pool.free(p) == 0
+    assert pool.free(p) != 0                          # second free of the same block
+    q = pool.alloc(2048)
+    assert pool.free(q + 512) != 0                    # not a block start
+    assert pool.L.ph_owns(pool.h, q)
+
+
+def test_free_null_and_foreign(pool):
+    assert pool.free(0) == 0
+    assert pool.log() == []
+    pool.L.ph_set_foreign_result(pool.h, 0)
+    assert pool.free(0x123456000) == 0
+    assert pool.log() == ["foreign %d" % 0x123456000]
+    assert pool.stats()["foreign_frees"] == 1
+
+
+# ------------------------------------------------------------------------------ churn invariants
+
+def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph):
+    pool = P(ph, capacity=8 * GiB)
+    rng = random.Random(4)
+    live = {}                                         # ptr -> rounded size
+    try:
+        for step in range(6000):
+            if live and (rng.random() < 0.45 or sum(live.values()) > 4 * GiB):
+                p = rng.choice(list(live))
+                assert pool.free(p) == 0
+                del live[p]
+            else:
+                n = int(4096 * 2 ** (rng.random() * 17))        # log-uniform 4 KiB .. 512 MiB
+                p = pool.alloc(n)
+                if p == 0:
+                    continue
+                rounded = (ph.ph_round_large(n) if n >= 8 * MiB else ph.ph_small_class_size(n))
+                assert p % (2 * MiB if n >= 8 * MiB else 512) == 0
+                assert p not in live
+                live[p] = rounded
+            if step % 500 == 0:
+                spans = sorted((p, p + n) for p, n in live.items())
+                assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "live blocks overlap"
+                st = pool.stats()
+                assert st["bytes_live"] == sum(live.values())
+                assert st["bytes_reserved"] == pool.L.ph_backing_used(pool.h)
+                assert st["bytes_live"] + st["bytes_cached_large"] + st["bytes_cached_small"] <= st["bytes_reserved"]
+        for p in list(live):
+            assert pool.free(p) == 0
+        st = pool.stats()
+        assert st["bytes_live"] == 0
+        pool.L.ph_release_unused(pool.h)
+        assert pool.L.ph_backing_used(pool.h) == 0 and pool.stats()["bytes_reserved"] == 0
+    finally:
+        pool.close()
