@@ -101,6 +101,9 @@ int sideaware_hash_mask(void);
 
 /* ---- additions (no counterpart in the reference) ---------------------------------------- */
 
+/* Upper bound on the device bytes the pool may hold (0 = none): a request that would pass it is
+ * answered like one the device refused (caches are given back, then null). */
+void sideaware_reserve_limit(size_t bytes);
 int sideaware_num_xcds(void);
 /* 1 when the start-up probe found workgroup i of a launch on XCD i % num_xcds. */
 int sideaware_xcd_dealing_verified(void);

@@ -26,6 +26,10 @@ struct DeviceGuard {
 // interior is handed out instead.
 void* HipBacking::acquire(size_t bytes) {
     DeviceGuard g(device_);
+    // The runtime may satisfy a request larger than the free device memory by spilling to host
+    // memory; a device pool must answer "out of memory" instead.
+    size_t free_bytes = 0, total_bytes = 0;
+    if (hipMemGetInfo(&free_bytes, &total_bytes) == hipSuccess && bytes > free_bytes) return nullptr;
     void* raw = nullptr;
     if (hipMalloc(&raw, bytes) != hipSuccess) {
         (void)hipGetLastError();      // an out-of-memory answer must not poison later calls

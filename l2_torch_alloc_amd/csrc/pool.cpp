@@ -61,6 +61,17 @@ void Pool::set_trim_thresholds(size_t start_bytes, size_t end_bytes) {
     trim_end_ = std::min(end_bytes, start_bytes);
 }
 
+void Pool::set_reserve_limit(size_t bytes) {
+    std::lock_guard<std::mutex> g(mu_);
+    reserve_limit_ = bytes;
+}
+
+void* Pool::backing_acquire_locked(size_t bytes) {
+    st_.backing_acquires++;
+    if (reserve_limit_ && st_.bytes_reserved + bytes > reserve_limit_) return nullptr;
+    return backing_->acquire(bytes);
+}
+
 void Pool::note_reserved(int64_t delta) {
     st_.bytes_reserved = (uint64_t)((int64_t)st_.bytes_reserved + delta);
     st_.peak_reserved = std::max(st_.peak_reserved, st_.bytes_reserved);
@@ -97,8 +108,7 @@ size_t Pool::trim_large_locked(size_t down_to) {
 }
 
 void* Pool::acquire_large_locked(size_t rounded, void* stream) {
-    void* p = backing_->acquire(rounded);
-    st_.backing_acquires++;
+    void* p = backing_acquire_locked(rounded);
     if (!p) return nullptr;
     assert(((uintptr_t)p % kRegionAlign) == 0);
     note_reserved((int64_t)rounded);
@@ -161,15 +171,13 @@ Pool::Slab* Pool::new_slab_locked(size_t block) {
     size_t want = std::min(std::max(block * 16, kRegionAlign), kMaxSlabBytes);
     want = std::max(want, block);
     size_t bytes = round_large(want);
-    void* p = backing_->acquire(bytes);
-    st_.backing_acquires++;
+    void* p = backing_acquire_locked(bytes);
     if (!p) {
         // the same ladder as the large path, compressed: drop caches, then retry once
         st_.ladder_retries++;
         trim_large_locked(0);
         release_empty_slabs_locked();
-        p = backing_->acquire(bytes);
-        st_.backing_acquires++;
+        p = backing_acquire_locked(bytes);
         if (!p) return nullptr;
     }
     note_reserved((int64_t)bytes);

@@ -81,6 +81,9 @@ public:
     void set_large_threshold(size_t bytes);
     size_t large_threshold() const { return large_threshold_; }
     void set_trim_thresholds(size_t start_bytes, size_t end_bytes);
+    // Upper bound on bytes held from the backing store (0 = none).  A request that would pass it
+    // walks the same ladder as one the device refused.
+    void set_reserve_limit(size_t bytes);
 
     // always_large: the reference's direct C entry points (sideaware_malloc and friends,
     // sideaware.cu:1280-1305) never take the small path.
@@ -130,6 +133,7 @@ private:
     Slab* new_slab_locked(size_t block);
     size_t trim_large_locked(size_t down_to);
     size_t release_empty_slabs_locked();
+    void* backing_acquire_locked(size_t bytes);
     void note_reserved(int64_t delta);
 
     Backing* backing_;
@@ -137,6 +141,7 @@ private:
     size_t large_threshold_ = 8ull << 20;
     size_t trim_start_ = 16ull << 30;
     size_t trim_end_ = 2ull << 30;
+    size_t reserve_limit_ = 0;
 
     std::unordered_map<size_t, std::vector<LargeBlock>> large_cache_;  // rounded size -> LIFO
     std::unordered_map<void*, LargeBlock> large_live_;

@@ -63,6 +63,7 @@ _SIGNATURES = {
     "sideaware_num_sm_side1": (_ci, []),
     "sideaware_min_sm_per_side": (_ci, []),
     "sideaware_hash_mask": (_ci, []),
+    "sideaware_reserve_limit": (None, [_sz]),
     "sideaware_num_xcds": (_ci, []),
     "sideaware_xcd_dealing_verified": (_ci, []),
     "sideaware_last_error": (ctypes.c_char_p, []),

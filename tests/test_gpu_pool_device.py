@@ -82,6 +82,23 @@ def test_out_of_memory_is_a_torch_exception_not_a_crash(sa):
     assert int(y.sum()) == 10 * MiB
 
 
+def test_reserve_limit_turns_into_torch_oom(sa):
+    lib = sa.library()
+    lib.sideaware_release_unused()
+    held = sa.sideaware_alloc_stats()["bytes_reserved"]
+    lib.sideaware_reserve_limit(held + 256 * MiB)
+    try:
+        ok = torch.empty(128 * MiB, dtype=torch.uint8, device="cuda")
+        with pytest.raises(torch.OutOfMemoryError):
+            torch.empty(512 * MiB, dtype=torch.uint8, device="cuda")
+        del ok
+    finally:
+        lib.sideaware_reserve_limit(0)
+        lib.sideaware_clear_error()
+    z = torch.empty(512 * MiB, dtype=torch.uint8, device="cuda")
+    assert z.data_ptr() % (2 * MiB) == 0
+
+
 def test_threshold_and_trim_settings_apply(sa):
     lib = sa.library()
     lib.sideaware_free_mapped_thresholds(32 * MiB, 0)

@@ -48,6 +48,7 @@ def ph():
     L.ph_release_unused.restype, L.ph_release_unused.argtypes = sz, [vp]
     L.ph_set_threshold.argtypes = [vp, sz]
     L.ph_set_trim.argtypes = [vp, sz, sz]
+    L.ph_set_limit.argtypes = [vp, sz]
     L.ph_owns.restype, L.ph_owns.argtypes = ctypes.c_int, [vp, u]
     L.ph_stats.restype, L.ph_stats.argtypes = ctypes.c_int, [vp, ctypes.POINTER(u), ctypes.c_int]
     L.ph_backing_used.restype, L.ph_backing_used.argtypes = sz, [vp]
@@ -215,6 +216,18 @@ def test_oom_ladder_and_null(ph):
         assert pool.alloc(44 * MiB) == c
     finally:
         pool.close()
+
+
+def test_reserve_limit_acts_like_a_full_device(pool):
+    pool.L.ph_set_limit(pool.h, 100 * MiB)
+    a = pool.alloc(60 * MiB)
+    assert a and pool.alloc(60 * MiB) == 0            # would hold 120 MiB
+    assert pool.stats()["failures"] == 1
+    pool.free(a)
+    b = pool.alloc(80 * MiB)                          # fits once the cached 60 MiB is given back
+    assert b and pool.stats()["bytes_reserved"] == 80 * MiB
+    pool.L.ph_set_limit(pool.h, 0)
+    assert pool.alloc(60 * MiB)
 
 
 def test_release_unused_returns_everything_cached(pool):
