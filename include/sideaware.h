@@ -110,8 +110,9 @@ int sideaware_xcd_dealing_verified(void);
 /* Text of the most recent failure on any thread ("" if none). */
 const char* sideaware_last_error(void);
 void sideaware_clear_error(void);
-/* Compiles header + template for gfx950 without touching a device. variant 0 = 32-bit indices
- * and 2 MiB-aligned base, 1 = 64-bit indices and any base.  Returns 0 on success; the compiler
+/* Compiles header + template for gfx950 without touching a device. variant bit 0: 0 = 32-bit indices
+ * (arrays below 2 GiB), 1 = 64-bit indices; bit 1: 0 = array fits the Infinity Cache, 1 = larger
+ * (everything streams).  Returns 0 on success; the compiler
  * log (possibly empty) is copied to `log`. */
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity);
 /* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */
@@ -124,8 +125,9 @@ const char* sideaware_config_block(int variant);
 int sideaware_kernel_info(int kernel_id, int variant, int* out);
 /* Pool counters, in the order of struct PoolStats (pool.h); returns the number written. */
 int sideaware_alloc_stats(unsigned long long* out, int capacity);
-/* Tuning knobs: "stripe_bytes", "nt_store", "groups_cap", "wg_threads", "shrink_grid".
- * Setting one drops every compiled kernel.  Returns 0 if the key is known. */
+/* Tuning knobs: "stripe_bytes", "slot_run", "groups_cap", "one_shot", "cache_bytes" (launch parameters) and
+ * "nt_store", "wg_threads" (compiled in: setting one drops every compiled kernel).
+ * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);
 

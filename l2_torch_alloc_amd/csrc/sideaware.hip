@@ -15,6 +15,7 @@
 
 #include "../../include/sideaware.h"
 #include "hip_backing.h"
+#include "launch_plan.h"
 #include "pool.h"
 #include "rtc.h"
 
@@ -29,7 +30,9 @@ static const char* kKernelTemplate =
     ;
 
 // Kernel id 0: a bit-exact copy, four bytes per element so that sixteen bytes make one vector.
-// The input is read with the streaming hint: a copy never reads its source twice.
+// No input is marked evict and UNROLLED is left at 1: one workgroup moves one 4 KiB chunk, the
+// source read plainly and the destination written with the streaming hint (both streaming once the
+// array no longer fits the Infinity Cache): the fastest combination measured on MI355X.
 static const char* kMemcpyHeader = R"SA_HDR(
 typedef int o0;
 typedef int i0;
@@ -37,7 +40,7 @@ struct unused {};
 typedef unused o1, o2, o3, i1, i2, i3;
 
 constexpr bool reverse_order = false;
-constexpr bool input_evict[4] = {true, false, false, false};
+constexpr bool input_evict[4] = {false, false, false, false};
 
 __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
                                                o0 &out0, o1 &out1, o2 &out2, o3 &out3,
@@ -70,11 +73,13 @@ static void set_error(const char* fmt, ...) {
 // ---------------------------------------------------------------------------------------------
 
 struct Tuning {
-    long long stripe_bytes = 16384;  // ownership stripe; the period (x8) must divide 2 MiB for the phase guarantee
-    long long nt_store = 1;          // outputs written with the nontemporal hint
+    long long stripe_bytes = 16384;  // ownership stripe of an XCD (power of two; shrunk for small arrays)
+    long long slot_run = 1;          // tiles a workgroup takes in a row; 0 = one contiguous block each
+    long long one_shot = 1;          // 1: one workgroup per tile unless the caller fixes the groups
+    long long cache_bytes = 256ll << 20;   // arrays larger than this are compiled to stream in both directions
+    long long nt_store = 2;          // nontemporal stores: 0 never, 1 always, 2 unless an input is marked evict
     long long groups_cap = 8;        // upper bound on default workgroups per CU
     long long wg_threads = 256;
-    long long shrink_grid = 1;       // launch fewer workgroups for arrays too small to feed them all
 };
 static Tuning g_tune;
 static std::atomic<unsigned> g_tune_generation{0};
@@ -89,20 +94,24 @@ static void load_tuning_from_env_once() {
     static std::once_flag once;
     std::call_once(once, [] {
         g_tune.stripe_bytes = env_ll("SIDEAWARE_STRIPE_BYTES", g_tune.stripe_bytes);
+        g_tune.slot_run = env_ll("SIDEAWARE_SLOT_RUN", g_tune.slot_run);
+        g_tune.one_shot = env_ll("SIDEAWARE_ONE_SHOT", g_tune.one_shot);
+        g_tune.cache_bytes = env_ll("SIDEAWARE_CACHE_BYTES", g_tune.cache_bytes);
         g_tune.nt_store = env_ll("SIDEAWARE_NT_STORE", g_tune.nt_store);
         g_tune.groups_cap = env_ll("SIDEAWARE_GROUPS_CAP", g_tune.groups_cap);
         g_tune.wg_threads = env_ll("SIDEAWARE_WG_THREADS", g_tune.wg_threads);
-        g_tune.shrink_grid = env_ll("SIDEAWARE_SHRINK_GRID", g_tune.shrink_grid);
     });
 }
 
 static long long* tune_slot(const char* key) {
     if (!key) return nullptr;
     if (!std::strcmp(key, "stripe_bytes")) return &g_tune.stripe_bytes;
+    if (!std::strcmp(key, "slot_run")) return &g_tune.slot_run;
+    if (!std::strcmp(key, "one_shot")) return &g_tune.one_shot;
+    if (!std::strcmp(key, "cache_bytes")) return &g_tune.cache_bytes;
     if (!std::strcmp(key, "nt_store")) return &g_tune.nt_store;
     if (!std::strcmp(key, "groups_cap")) return &g_tune.groups_cap;
     if (!std::strcmp(key, "wg_threads")) return &g_tune.wg_threads;
-    if (!std::strcmp(key, "shrink_grid")) return &g_tune.shrink_grid;
     return nullptr;
 }
 
@@ -278,6 +287,8 @@ struct CompiledKernel {
     hipFunction_t fn = nullptr;
     int vgprs = 0, sgprs = 0;
     int occupancy = 0;          // workgroups per CU the hardware can hold
+    int tile_vectors = 0;       // from the module's sideaware_kernel_meta
+    int owner_is_o0 = 0;
     bool failed = false;
     unsigned generation = 0;
 };
@@ -285,7 +296,7 @@ struct CompiledKernel {
 struct KernelEntry {
     std::string header;
     int default_groups = 0;     // 0: decide from occupancy
-    std::vector<CompiledKernel> compiled;   // [device * 2 + variant]
+    std::vector<CompiledKernel> compiled;   // [device * 4 + variant]; variant = 2*beyond_cache + wide_index
 };
 
 static std::mutex g_kernels_mu;
@@ -304,13 +315,13 @@ static std::string config_block(int variant, int num_xcds, int num_cus) {
     std::string s;
     s += "#define SA_NUM_XCD " + std::to_string(num_xcds) + "\n";
     s += "#define SA_WG_THREADS " + std::to_string(g_tune.wg_threads) + "\n";
-    s += "#define SA_STRIPE_BYTES " + std::to_string(g_tune.stripe_bytes) + "\n";
     s += "#define SA_NT_STORE " + std::to_string(g_tune.nt_store) + "\n";
     // Names the reference injects (sideaware.cu:789-794); kept so headers that mention them compile.
     s += "#define MAX_SM " + std::to_string(num_cus) + "\n";
     s += "#define HASH " + std::to_string((stripe_hash_mask(num_xcds) | (1 << 21)) / 16) + "\n";
-    s += variant ? "using size_type = long long;\nconstexpr bool aligned_2MiB = false;\n"
-                 : "using size_type = int;\nconstexpr bool aligned_2MiB = true;\n";
+    s += "#define SA_BEYOND_CACHE " + std::to_string((variant >> 1) & 1) + "\n";
+    s += (variant & 1) ? "using size_type = long long;\nconstexpr bool aligned_2MiB = false;\n"
+                       : "using size_type = int;\nconstexpr bool aligned_2MiB = true;\n";
     return s;
 }
 
@@ -328,7 +339,7 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
         return nullptr;
     }
     KernelEntry& e = *g_kernels[kernel_id];
-    size_t slot = (size_t)ctx->device * 2 + (variant ? 1 : 0);
+    size_t slot = (size_t)ctx->device * 4 + (size_t)(variant & 3);
     if (e.compiled.size() <= slot) e.compiled.resize(slot + 1);
     CompiledKernel& k = e.compiled[slot];
     unsigned gen = g_tune_generation.load();
@@ -356,6 +367,24 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
         set_error("kernel %d (variant %d) failed to load: %s", kernel_id, variant, hipGetErrorString(err));
         (void)hipGetLastError();
         return nullptr;
+    }
+    // The instantiation says how many vectors make a tile and which array's address defines
+    // ownership; the launch planner needs both.
+    {
+        hipDeviceptr_t meta_ptr = nullptr;
+        size_t meta_bytes = 0;
+        int meta[4] = {0, 0, 0, 0};
+        err = hipModuleGetGlobal(&meta_ptr, &meta_bytes, k.module, "sideaware_kernel_meta");
+        if (err == hipSuccess && meta_bytes >= sizeof meta) err = hipMemcpyDtoH(meta, meta_ptr, sizeof meta);
+        if (err != hipSuccess || meta[0] <= 0) {
+            k.failed = true;
+            k.fn = nullptr;
+            set_error("kernel %d (variant %d): cannot read its tile size: %s", kernel_id, variant, hipGetErrorString(err));
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        k.tile_vectors = meta[0];
+        k.owner_is_o0 = meta[2];
     }
     (void)hipFuncGetAttribute(&k.vgprs, HIP_FUNC_ATTRIBUTE_NUM_REGS, k.fn);
     int occ = 0;
@@ -456,8 +485,7 @@ int sideaware_create_kernel_advanced(const char* header, bool precompile, int de
     int id = register_header(header, default_num_groups);
     if (precompile) {
         if (DeviceContext* ctx = get_context()) {
-            get_kernel(ctx, id, 0);
-            get_kernel(ctx, id, 1);
+            for (int v = 0; v < 4; v++) get_kernel(ctx, id, v);
         }
     }
     return id;
@@ -482,11 +510,12 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         return;
     }
 
-    // 32-bit indices and the base-free stripe phase need a 2 MiB-aligned base and < 2 GiB
-    // (sideaware.cu:1386-1388); everything else takes the general variant.
-    const bool misaligned = ((uintptr_t)in0 % kRegionAlign) || ((uintptr_t)out0 % kRegionAlign);
-    const bool wide = num_bytes >= (2ull << 30);
-    const int variant = (misaligned || wide) ? 1 : 0;
+    // Two instantiations per op: 32-bit indices below 2 GiB, 64-bit from there on (the reference
+    // also sends bases that are not 2 MiB-aligned to its 64-bit variant, sideaware.cu:1386-1388;
+    // here the base only shifts the planner's b0, whatever its alignment).
+    // and, independently, one pair for arrays that fit the Infinity Cache and one for larger ones.
+    const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
+    const int variant = wide | (num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0);
 
     CompiledKernel* k = get_kernel(ctx, kernel_id, variant);
     if (!k) return;
@@ -496,31 +525,39 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         std::lock_guard<std::mutex> g(g_kernels_mu);
         default_groups = g_kernels[kernel_id]->default_groups;
     }
-    int groups = parallel_groups > 0 ? parallel_groups : default_groups;
-    if (groups <= 0) {
-        groups = k->occupancy > 0 ? k->occupancy : 4;
-        if (groups > g_tune.groups_cap) groups = (int)g_tune.groups_cap;
-    }
+    // Workgroups per XCD.  The caller's parallel_groups / forced_per_side, or the header's
+    // default, fix a persistent grid of (CUs per XCD) x groups; otherwise the tuning decides
+    // between one workgroup per tile and a persistent grid sized from the kernel's occupancy.
     int per_xcd = ctx->cus_per_xcd;
     if (forced_per_side > 0 && forced_per_side < per_xcd) per_xcd = forced_per_side;
-    long long slots = (long long)per_xcd * groups;
+    int groups = parallel_groups > 0 ? parallel_groups : default_groups;
+    long long slots_wanted;
+    if (groups > 0 || forced_per_side > 0 || !g_tune.one_shot) {
+        if (groups <= 0) {
+            groups = k->occupancy > 0 ? k->occupancy : 4;
+            if (groups > g_tune.groups_cap) groups = (int)g_tune.groups_cap;
+        }
+        slots_wanted = (long long)per_xcd * groups;
+    } else {
+        slots_wanted = 0;
+    }
 
     const long long num_vectors = (long long)(num_bytes / 16);
-    if (g_tune.shrink_grid) {
-        // An upper bound on the tiles any XCD can own (tiles are at least one chunk, and an
-        // unaligned base shifts the first stripe period): workgroups beyond it would find no work.
-        long long chunks = (num_vectors + g_tune.wg_threads - 1) / g_tune.wg_threads;
-        long long most = chunks / ctx->num_xcds + 2;
-        if (slots > most) slots = most;
-    }
-    if (slots < 1) slots = 1;
-    const unsigned grid = (unsigned)(slots * ctx->num_xcds);
+    // The ownership stripe: the tuned size, shrunk for arrays too short to give every XCD at least
+    // ~32 stripes of it (one XCD can be a stripe ahead of another).
+    unsigned long long stripe = (unsigned long long)g_tune.stripe_bytes;
+    while (stripe > 4096 && stripe * 32 * ctx->num_xcds > num_bytes) stripe >>= 1;
+    const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0);
+    LaunchPlan plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds, stripe,
+                                  g_tune.slot_run, slots_wanted);
+    const unsigned grid = plan.grid;
 
-    long long nv64 = num_vectors;
-    int nv32 = (int)num_vectors;
+    long long nv64 = num_vectors, ft64 = plan.full_tiles, b064 = plan.b0, uc64 = plan.u_count, run64 = plan.run;
+    int nv32 = (int)num_vectors, ft32 = (int)plan.full_tiles, b032 = (int)plan.b0, uc32 = (int)plan.u_count,
+        run32 = (int)plan.run;
     int* mem = (int*)sideband_memory;
-    void* args[11];
-    args[0] = variant ? (void*)&nv64 : (void*)&nv32;
+    void* args[17];
+    args[0] = wide ? (void*)&nv64 : (void*)&nv32;
     args[1] = &out0;
     args[2] = &out1;
     args[3] = &out2;
@@ -531,6 +568,12 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     args[8] = &in3;
     args[9] = &mem;
     args[10] = &sideband_value;
+    args[11] = wide ? (void*)&ft64 : (void*)&ft32;
+    args[12] = wide ? (void*)&b064 : (void*)&b032;
+    args[13] = wide ? (void*)&uc64 : (void*)&uc32;
+    args[14] = wide ? (void*)&run64 : (void*)&run32;
+    args[15] = &plan.r;
+    args[16] = &plan.tail_block;
 
     ScopedDevice guard(ctx->device);
     hipError_t err = hipModuleLaunchKernel(k->fn, grid, 1, 1, (unsigned)g_tune.wg_threads, 1, 1, 0,
@@ -646,7 +689,7 @@ void sideaware_clear_error(void) {
 
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity) {
     std::string hdr = header && *header ? header : kMemcpyHeader;
-    CompileResult r = compile_for_gfx950(full_source(hdr, variant ? 1 : 0, kDefaultXcds, kDefaultCUs));
+    CompileResult r = compile_for_gfx950(full_source(hdr, variant & 3, kDefaultXcds, kDefaultCUs));
     if (log && log_capacity) {
         std::snprintf(log, log_capacity, "%s", r.log.c_str());
     }
@@ -658,16 +701,16 @@ const char* sideaware_memcpy_header(void) { return kMemcpyHeader; }
 
 const char* sideaware_config_block(int variant) {
     static std::mutex mu;
-    static std::string text[2];
+    static std::string text[4];
     std::lock_guard<std::mutex> g(mu);
-    text[variant ? 1 : 0] = config_block(variant ? 1 : 0, kDefaultXcds, kDefaultCUs);
-    return text[variant ? 1 : 0].c_str();
+    text[variant & 3] = config_block(variant & 3, kDefaultXcds, kDefaultCUs);
+    return text[variant & 3].c_str();
 }
 
 int sideaware_kernel_info(int kernel_id, int variant, int* out) {
     DeviceContext* ctx = get_context();
     if (!ctx || !out) return 1;
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant ? 1 : 0);
+    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & 3);
     if (!k) return 1;
     int groups;
     {
@@ -701,10 +744,12 @@ int sideaware_tune(const char* key, long long value) {
     long long* slot = tune_slot(key);
     if (!slot) return 1;
     if (!std::strcmp(key, "wg_threads") && (value < 64 || value > 1024 || (value & (value - 1)))) return 1;
-    if (!std::strcmp(key, "stripe_bytes") && (value < 4096 || (value & (value - 1)))) return 1;
+    if (!std::strcmp(key, "stripe_bytes") && (value < 4096 || value > (1ll << 30) || (value & (value - 1)))) return 1;
+    if (!std::strcmp(key, "slot_run") && (value < 0 || value > (1 << 20))) return 1;
     if (*slot != value) {
         *slot = value;
-        g_tune_generation++;       // compiled kernels are rebuilt on their next use
+        const bool compiled_in = !std::strcmp(key, "nt_store") || !std::strcmp(key, "wg_threads");
+        if (compiled_in) g_tune_generation++;      // compiled kernels are rebuilt on their next use
     }
     return 0;
 }

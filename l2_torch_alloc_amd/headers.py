@@ -27,7 +27,7 @@ def memcpy_header() -> bytes:
     return (
         "typedef int o0;\ntypedef int i0;\n" + _UNUSED +
         "typedef unused o1, o2, o3, i1, i2, i3;\n"
-        "constexpr bool reverse_order = false;\n" + _evict([True]) +
+        "constexpr bool reverse_order = false;\n" + _evict([False]) +
         "__device__ void elementwise_op(size_t element_idx, int sideband,\n"
         "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
         "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {\n"
@@ -44,7 +44,7 @@ _ROPE_TYPES = {
 
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
                 layout: str = "qkv", backward: bool = False, unrolled: int | None = None,
-                reverse_order: bool = False) -> bytes:
+                reverse_order: bool = False, evict_input: bool = False) -> bytes:
     """RoPE forward (or backward) in place or out of place.
 
     layout "qkv":   one tensor (B, T, n_q + 2*n_kv, head_dim); q and k heads are rotated, the
@@ -78,7 +78,10 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     if unrolled is not None:
         lines.append("#define UNROLLED %d\n" % unrolled)
     lines.append("constexpr bool reverse_order = %s;\n" % ("true" if reverse_order else "false"))
-    lines.append(_evict([True, False]))      # activations stream; the table is re-read and stays cached
+    # The table is re-read by every head of a token and must stay cached.  The activations are
+    # read once: either they are read with the streaming hint (evict_input) or, by default,
+    # written with it.
+    lines.append(_evict([evict_input, False]))
     lines.append(
         "constexpr int rope_T = %d;\n"
         "constexpr int rope_half = %d;          // pairs per head\n"
@@ -116,13 +119,13 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     return "".join(lines).encode()
 
 
-def scale_bias_bf16_header(unrolled: int | None = None) -> bytes:
+def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = False) -> bytes:
     """bf16 ``y = x*scale + bias``; scale and bias are two fp32 values read from the sideband
     pointer at launch, so one compiled kernel serves every (scale, bias)."""
     lines = ["typedef __bf16 o0;\ntypedef __bf16 i0;\n", _UNUSED, "typedef unused o1, o2, o3, i1, i2, i3;\n"]
     if unrolled is not None:
         lines.append("#define UNROLLED %d\n" % unrolled)
-    lines.append("constexpr bool reverse_order = false;\n" + _evict([True]))
+    lines.append("constexpr bool reverse_order = false;\n" + _evict([evict_input]))
     lines.append(
         "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
         "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"

@@ -1,5 +1,6 @@
 // Appended after the kernel template: runs the whole grid on the CPU, lane by lane, and checks
-// the result.  stdin carries one case per line: "grid num_vectors base_offset_bytes".
+// the result.  stdin carries one case per line:
+// "grid num_vectors base_offset_bytes stripe_log2 slot_run".
 //
 // Every array is a posix_memalign block of exactly the bytes it needs, 2 MiB-aligned and then
 // shifted by base_offset, so a lane that reads or writes past the end trips AddressSanitizer
@@ -12,15 +13,27 @@
 #include <cstdio>
 #include <cstdlib>
 
+#include "../../l2_torch_alloc_amd/csrc/launch_plan.h"
+
+static unsigned g_stripe_log2 = 14, g_slot_run = 1;
+
+// `grid` is the caller's wish, as the launcher's parallel_groups would be: a persistent grid of
+// that many workgroups (rounded to whole XCDs), or 0 for one workgroup per tile.  The plan is made
+// by the same function the launcher uses.
 static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3* o3,
                      const vi0* i0, const vi1* i1, const vi2* i2, const vi3* i3, int* mem, int val) {
-    gridDim = {grid, 1, 1};
+    const unsigned long long base = sideaware_kernel_meta[2] ? (unsigned long long)o0 : (unsigned long long)i0;
+    sideaware::LaunchPlan p = sideaware::plan_launch(base, (long long)nv, sideaware_kernel_meta[0], SA_NUM_XCD,
+                                                     1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
+    gridDim = {p.grid, 1, 1};
     blockDim = {SA_WG_THREADS, 1, 1};
-    for (unsigned b = 0; b < grid; b++) {
+    for (unsigned b = 0; b < p.grid; b++) {
         for (unsigned t = 0; t < SA_WG_THREADS; t++) {
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
-            sideaware_elementwise(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val);
+            sideaware_elementwise(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val,
+                                  (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
+                                  p.r, p.tail_block);
         }
     }
 }
@@ -130,12 +143,13 @@ int main() {
     long long nv;
     size_t off;
     int cases = 0, failed = 0;
-    while (std::scanf("%u %lld %zu", &grid, &nv, &off) == 3) {
+    while (std::scanf("%u %lld %zu %u %u", &grid, &nv, &off, &g_stripe_log2, &g_slot_run) == 5) {
         cases++;
         int bad = run_case(grid, nv, off);
         if (bad) {
             failed++;
-            std::printf("FAIL grid=%u nv=%lld off=%zu: %d bad elements\n", grid, nv, off, bad);
+            std::printf("FAIL grid=%u nv=%lld off=%zu stripe_log2=%u run=%u: %d bad elements\n", grid, nv, off,
+                        g_stripe_log2, g_slot_run, bad);
         }
     }
     std::printf("cases=%d failed=%d\n", cases, failed);

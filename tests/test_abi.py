@@ -93,9 +93,17 @@ def test_tuning_knobs(lib):
     old = lib.sideaware_tune_get(b"stripe_bytes")
     assert lib.sideaware_tune(b"stripe_bytes", 65536) == 0
     assert lib.sideaware_tune_get(b"stripe_bytes") == 65536
-    assert b"#define SA_STRIPE_BYTES 65536" in lib.sideaware_config_block(0)
-    assert b"using size_type = long long" in lib.sideaware_config_block(1)
     assert lib.sideaware_tune(b"stripe_bytes", old) == 0
+    assert lib.sideaware_tune(b"slot_run", 0) == 0 and lib.sideaware_tune_get(b"slot_run") == 0
+    assert lib.sideaware_tune(b"slot_run", 1) == 0
+    assert b"using size_type = long long" in lib.sideaware_config_block(1)
+    assert b"using size_type = int;" in lib.sideaware_config_block(0)
+    assert b"#define SA_BEYOND_CACHE 0" in lib.sideaware_config_block(1)
+    assert b"#define SA_BEYOND_CACHE 1" in lib.sideaware_config_block(2)
+    old_nt = lib.sideaware_tune_get(b"nt_store")
+    assert lib.sideaware_tune(b"nt_store", 0) == 0
+    assert b"#define SA_NT_STORE 0" in lib.sideaware_config_block(0)
+    assert lib.sideaware_tune(b"nt_store", old_nt) == 0
 
 
 def compile_ok(lib, header, variant):
@@ -120,7 +128,7 @@ SHIPPED_HEADERS = {
 
 
 @pytest.mark.parametrize("name", sorted(SHIPPED_HEADERS))
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 def test_shipped_headers_compile_for_gfx950(lib, name, variant):
     rc, log = compile_ok(lib, SHIPPED_HEADERS[name], variant)
     assert rc == 0, log
@@ -149,7 +157,7 @@ constexpr bool input_evict[4] = {1,1,1,1};
 """
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 3])
 def test_cuda_dialect_header_compiles(lib, variant):
     rc, log = compile_ok(lib, CUDA_DIALECT_HEADER, variant)
     assert rc == 0, log

@@ -71,27 +71,42 @@ def test_release_unused_gives_memory_back(sa):
     assert sa.sideaware_alloc_stats()["bytes_cached_large"] == 0
 
 
-def test_out_of_memory_is_a_torch_exception_not_a_crash(sa):
+def test_out_of_memory_is_a_null_pointer_not_a_crash(sa):
+    # More than the device holds: every step of the ladder fails and the entry point returns null
+    # (sideaware.cu:1250-1251 ends the same way).  PyTorch's pluggable-allocator shim does not check
+    # the pointer, so the tensor it builds has a null data pointer; it is never touched here.
     total = torch.cuda.get_device_properties(0).total_memory
-    with pytest.raises(torch.OutOfMemoryError):
-        torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
-    assert sa.sideaware_alloc_stats()["failures"] >= 1
-    sa.library().sideaware_clear_error()
+    lib = sa.library()
+    before = sa.sideaware_alloc_stats()["failures"]
+    p = lib.sideaware_malloc_auto(total + (8 << 30), 0, None)
+    assert p is None
+    assert sa.sideaware_alloc_stats()["failures"] == before + 1
+    t = torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
+    assert t.data_ptr() == 0
+    del t
+    out = ctypes.c_void_p(1)
+    assert lib.sideaware_malloc(ctypes.byref(out), total + (8 << 30)) == 2      # hipErrorOutOfMemory
+    assert out.value is None
+    lib.sideaware_clear_error()
     # and the pool still serves requests afterwards
     y = torch.ones(10 * MiB, dtype=torch.uint8, device="cuda")
     assert int(y.sum()) == 10 * MiB
 
 
-def test_reserve_limit_turns_into_torch_oom(sa):
+def test_reserve_limit_acts_like_a_full_device(sa):
     lib = sa.library()
     lib.sideaware_release_unused()
     held = sa.sideaware_alloc_stats()["bytes_reserved"]
     lib.sideaware_reserve_limit(held + 256 * MiB)
     try:
-        ok = torch.empty(128 * MiB, dtype=torch.uint8, device="cuda")
-        with pytest.raises(torch.OutOfMemoryError):
-            torch.empty(512 * MiB, dtype=torch.uint8, device="cuda")
-        del ok
+        ok = lib.sideaware_malloc_auto(128 * MiB, 0, None)
+        assert ok and ok % (2 * MiB) == 0
+        assert lib.sideaware_malloc_auto(512 * MiB, 0, None) is None
+        lib.sideaware_free_auto(ok, 128 * MiB, 0, None)
+        # with the cached 128 MiB given back by the ladder, 200 MiB fits under the limit
+        again = lib.sideaware_malloc_auto(200 * MiB, 0, None)
+        assert again
+        lib.sideaware_free_auto(again, 200 * MiB, 0, None)
     finally:
         lib.sideaware_reserve_limit(0)
         lib.sideaware_clear_error()

@@ -2,8 +2,8 @@
 
 The text comes out of the built library (``sideaware_kernel_source`` / ``sideaware_config_block``),
 so what is checked is exactly what hipRTC compiles on the GPU box.  For each compile-time
-configuration (index width, UNROLLED, ownership stripe, traversal order) a small driver is built
-with the ROCm clang as plain host C++ and fed many (grid, length, base offset) cases: the
+configuration (index width, UNROLLED, traversal order) a small driver is built with the ROCm
+clang as plain host C++ and fed many (grid, length, base offset, stripe, run) cases: the
 workgroup -> tile map must visit every 16-byte vector exactly once, never touch a byte outside
 the arrays, and do so for any grid size, which is the property the reference could not offer
 (its map skips data unless exactly one block runs per SM, sideaware.cu:211-212).
@@ -68,8 +68,7 @@ def lib():
     return L
 
 
-def build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse, header=None):
-    assert lib.sideaware_tune(b"stripe_bytes", stripe) == 0
+def build_driver(lib, tmp_path, case, variant, unrolled, reverse, header=None):
     config = lib.sideaware_config_block(variant).decode()
     template = lib.sideaware_kernel_source().decode()
     if header is None:
@@ -83,8 +82,7 @@ def build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse, header
         "#define SA_CASE_%s 1" % case,
         '#include "%s"' % os.path.join(NATIVE, "kernel_cpu_driver.h"),
     ])
-    src = tmp_path / ("tu_%s_v%d_u%s_s%d_r%d_%x.cpp" % (case, variant, unrolled, stripe, reverse,
-                                                        hash(header) & 0xffffff))
+    src = tmp_path / ("tu_%s_v%d_u%s_r%d_%x.cpp" % (case, variant, unrolled, reverse, hash(header) & 0xffffff))
     exe = str(src)[:-4]
     src.write_text(tu)
     cmd = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
@@ -100,40 +98,42 @@ def cases_for(variant, unrolled, rng):
     lengths |= {rng.randrange(0, 70 * tile) for _ in range(40)}
     # every residue class of the tail for one tile count, sampled
     lengths |= {5 * tile + r for r in rng.sample(range(tile), 24)}
-    grids = [8, 16, 24, 56, 8 * 37, 2048]
-    offsets = [0] if variant == 0 else [0, 16, 4096, 16384 + 32, 3 * 65536 + 4096 + 48, (2 << 20) - 16]
+    grids = [0, 8, 16, 24, 56, 8 * 37, 2048]       # 0: one workgroup per tile
+    offsets = [0, 16, 4096, 16384 + 32, 3 * 65536 + 4096 + 48, (2 << 20) - 16]
+    stripes = [12, 14, 16, 18, 21, 24]          # log2 bytes: 4 KiB .. 16 MiB
+    runs = [0, 1, 2, 3, 16, 1000]               # 0 = one contiguous block per workgroup
     out = []
     for n in sorted(lengths):
         for g in rng.sample(grids, 2):
-            for off in rng.sample(offsets, min(2, len(offsets))):
-                out.append((g, n, off))
+            for off in rng.sample(offsets, 2):
+                out.append((g, n, off, rng.choice(stripes), rng.choice(runs)))
     return out
 
 
 CONFIGS = [
-    # case, variant, UNROLLED (None = template default), stripe bytes, reverse_order
-    ("INCREMENT", 0, None, 16384, False),
-    ("INCREMENT", 1, None, 16384, False),
-    ("INCREMENT", 0, 1, 4096, True),
-    ("INCREMENT", 1, 2, 65536, True),
-    ("INCREMENT", 1, 3, 16384, False),      # tile is not a power of two
-    ("INCREMENT", 0, 8, 4096, False),       # tile larger than the stripe
-    ("INCREMENT", 1, 4, 262144, True),      # largest stripe with the 2 MiB phase guarantee
-    ("MIXED", 0, None, 16384, False),
-    ("MIXED", 1, 2, 4096, True),
+    # case, variant (0: 32-bit indices, 1: 64-bit), UNROLLED (None = template default), reverse_order
+    ("INCREMENT", 0, None, False),
+    ("INCREMENT", 1, None, False),
+    ("INCREMENT", 0, 1, True),
+    ("INCREMENT", 1, 2, True),
+    ("INCREMENT", 1, 3, False),      # tile is not a power of two
+    ("INCREMENT", 0, 8, False),      # tile larger than the smallest stripe
+    ("INCREMENT", 0, 2, False),      # the built-in copy's setting
+    ("MIXED", 0, None, False),
+    ("MIXED", 1, 2, True),
 ]
 
 
-@pytest.mark.parametrize("case,variant,unrolled,stripe,reverse", CONFIGS)
-def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, stripe, reverse):
+@pytest.mark.parametrize("case,variant,unrolled,reverse", CONFIGS)
+def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, reverse):
     if not os.path.exists(CLANG):
         pytest.skip("ROCm clang++ not found")
-    exe = build_driver(lib, tmp_path, case, variant, unrolled, stripe, reverse)
-    rng = random.Random(hash((case, variant, unrolled, stripe, reverse)) & 0xffff)
+    exe = build_driver(lib, tmp_path, case, variant, unrolled, reverse)
+    rng = random.Random(hash((case, variant, unrolled, reverse)) & 0xffff)
     cases = cases_for(variant, unrolled, rng)
     if case == "MIXED":
-        cases = [(g, n, off - off % 64) for (g, n, off) in cases]   # halves of the offset stay 16 B-aligned
-    text = "".join("%d %d %d\n" % c for c in cases)
+        cases = [(g, n, off - off % 64, s, r) for (g, n, off, s, r) in cases]   # halved offsets stay 16 B-aligned
+    text = "".join("%d %d %d %d %d\n" % c for c in cases)
     proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
                           env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
@@ -157,7 +157,7 @@ def test_rope_headers_on_cpu(lib, tmp_path, T, n_q, n_kv, head_dim, dtype, layou
         pytest.skip("ROCm clang++ not found")
     from l2_torch_alloc_amd import headers
     header = headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout).decode()
-    exe = build_driver(lib, tmp_path, "ROPE", variant, None, 16384, False, header=header)
+    exe = build_driver(lib, tmp_path, "ROPE", variant, None, False, header=header)
     heads = n_q + 2 * n_kv if layout == "qkv" else n_q
     pair_bytes = 8 if dtype == "fp32" else 4
     vecs_per_token = heads * (head_dim // 2) * pair_bytes // 16
@@ -165,11 +165,11 @@ def test_rope_headers_on_cpu(lib, tmp_path, T, n_q, n_kv, head_dim, dtype, layou
     cases = []
     for tokens in (1, T - 1, T, T + 1, 3 * T, 7 * T + 2):
         nv = tokens * vecs_per_token
-        for grid in rng.sample([8, 16, 56, 2048], 2):
-            for off in ([0] if variant == 0 else [0, 16, 4096 + 32]):
-                cases.append((grid, nv, off))
-    cases.append((8, 3 * vecs_per_token + 1, 0))       # length that is not a whole number of tokens
-    text = "".join("%d %d %d\n" % c for c in cases)
+        for grid in rng.sample([0, 8, 16, 56, 2048], 2):
+            for off in (0, 16, 4096 + 32):
+                cases.append((grid, nv, off, rng.choice([12, 14, 18, 22]), rng.choice([0, 1, 4])))
+    cases.append((8, 3 * vecs_per_token + 1, 0, 14, 1))   # length that is not a whole number of tokens
+    text = "".join("%d %d %d %d %d\n" % c for c in cases)
     proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
                           env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
