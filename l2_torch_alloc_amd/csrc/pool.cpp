@@ -124,19 +124,23 @@ void* Pool::acquire_large_locked(size_t rounded, void* stream) {
 void* Pool::allocate_large_locked(size_t bytes, void* stream) {
     const size_t rounded = round_large(bytes);
 
-    // 1) exact-size reuse, newest first (sideaware.cu:1199-1219)
-    auto it = large_cache_.find(rounded);
-    if (it != large_cache_.end() && !it->second.empty()) {
+    // 1) exact-size reuse, newest first (sideaware.cu:1199-1219); failing that, the smallest
+    //    cached region that is at most one eighth larger, handed out whole.  Any 2 MiB-aligned
+    //    region serves, and a driver allocation costs hundreds of microseconds.
+    auto it = large_cache_.lower_bound(rounded);
+    while (it != large_cache_.end() && it->second.empty()) ++it;
+    if (it != large_cache_.end() && it->first <= rounded + rounded / 8) {
         LargeBlock blk = it->second.back();
         it->second.pop_back();
-        st_.bytes_cached_large -= rounded;
+        if (it->second.empty()) large_cache_.erase(it);
+        st_.bytes_cached_large -= blk.bytes;
         if (blk.last_stream != stream) {
             backing_->sync_stream(blk.last_stream);
             st_.stream_syncs++;
             blk.last_stream = stream;
         }
         large_live_.emplace(blk.ptr, blk);
-        st_.bytes_live += rounded;
+        st_.bytes_live += blk.bytes;
         st_.large_hits++;
         return blk.ptr;
     }
@@ -335,6 +339,18 @@ size_t Pool::release_unused() {
 PoolStats Pool::stats() {
     std::lock_guard<std::mutex> g(mu_);
     return st_;
+}
+
+size_t Pool::block_bytes(void* ptr) {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = large_live_.find(ptr);
+    if (it != large_live_.end()) return it->second.bytes;
+    auto sit = slab_by_page_.find((uintptr_t)ptr / kRegionAlign);
+    if (sit == slab_by_page_.end()) return 0;
+    Slab* slab = sit->second;
+    size_t off = (char*)ptr - slab->base;
+    bool live = off % slab->block == 0 && off / slab->block < slab->carved && slab->in_use[off / slab->block];
+    return live ? slab->block : 0;
 }
 
 bool Pool::owns_live(void* ptr) {

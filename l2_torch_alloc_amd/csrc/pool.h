@@ -11,8 +11,9 @@
 // caching behaviour:
 //
 //   large  (size >= threshold): dedicated region, size rounded up to 2 MiB, exact-size LIFO
-//          reuse cache, trimmed back to the backing store when it outgrows the thresholds,
-//          and the reference's four-step out-of-memory ladder (sideaware.cu:1233-1252);
+//          reuse cache (then the smallest cached region at most 1/8 larger, handed out whole),
+//          trimmed back to the backing store when it outgrows the thresholds, and the
+//          reference's four-step out-of-memory ladder (sideaware.cu:1233-1252);
 //   small  (size <  threshold): 512 B-granular size classes carved from slabs, so the common
 //          small request never reaches the driver (the reference forwards these to
 //          cudaMallocAsync, sideaware.cu:1326-1339).
@@ -24,6 +25,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <unordered_map>
@@ -51,7 +53,7 @@ public:
 };
 
 struct PoolStats {
-    uint64_t large_hits = 0;        // large requests served from the reuse cache
+    uint64_t large_hits = 0;        // large requests served from the reuse cache (exact or near fit)
     uint64_t large_misses = 0;      // large requests that went to the backing store
     uint64_t small_hits = 0;        // small requests served from a class free list
     uint64_t small_carves = 0;      // small requests carved from a slab's untouched tail
@@ -97,6 +99,8 @@ public:
     PoolStats stats();
     // For the property tests: true when `ptr` is a live block of this pool.
     bool owns_live(void* ptr);
+    // Bytes actually held by the live block at `ptr` (0 if it is not one).
+    size_t block_bytes(void* ptr);
 
     static size_t round_large(size_t bytes);
     static size_t small_class_size(size_t bytes);   // rounded size of a small request
@@ -143,7 +147,7 @@ private:
     size_t trim_end_ = 2ull << 30;
     size_t reserve_limit_ = 0;
 
-    std::unordered_map<size_t, std::vector<LargeBlock>> large_cache_;  // rounded size -> LIFO
+    std::map<size_t, std::vector<LargeBlock>> large_cache_;            // rounded size -> LIFO, sizes ordered
     std::unordered_map<void*, LargeBlock> large_live_;
     std::vector<SmallClass> small_;                                    // class index -> state
     std::unordered_map<uintptr_t, Slab*> slab_by_page_;                // addr >> 21 -> slab

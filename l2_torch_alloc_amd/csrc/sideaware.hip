@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cctype>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -34,6 +35,7 @@ static const char* kKernelTemplate =
 // source read plainly and the destination written with the streaming hint (both streaming once the
 // array no longer fits the Infinity Cache): the fastest combination measured on MI355X.
 static const char* kMemcpyHeader = R"SA_HDR(
+#define KERNEL_NAME sideaware_copy
 typedef int o0;
 typedef int i0;
 struct unused {};
@@ -295,6 +297,7 @@ struct CompiledKernel {
 
 struct KernelEntry {
     std::string header;
+    std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`
     int default_groups = 0;     // 0: decide from occupancy
     std::vector<CompiledKernel> compiled;   // [device * 4 + variant]; variant = 2*beyond_cache + wide_index
 };
@@ -303,10 +306,23 @@ static std::mutex g_kernels_mu;
 static std::vector<std::unique_ptr<KernelEntry>> g_kernels;
 static std::unordered_map<std::string, int> g_header_to_id;
 
+// Finds `#define KERNEL_NAME identifier` in an op header.
+static std::string kernel_name_of(const std::string& header) {
+    const std::string key = "#define KERNEL_NAME";
+    size_t pos = header.find(key);
+    if (pos == std::string::npos) return "sideaware_elementwise";
+    pos += key.size();
+    while (pos < header.size() && (header[pos] == ' ' || header[pos] == '\t')) pos++;
+    size_t end = pos;
+    while (end < header.size() && (std::isalnum((unsigned char)header[end]) || header[end] == '_')) end++;
+    return end > pos ? header.substr(pos, end - pos) : "sideaware_elementwise";
+}
+
 static void ensure_builtin_locked() {
     if (!g_kernels.empty()) return;
     auto e = std::make_unique<KernelEntry>();
     e->header = kMemcpyHeader;
+    e->function_name = kernel_name_of(e->header);
     g_kernels.push_back(std::move(e));
 }
 
@@ -360,7 +376,7 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
     }
     ScopedDevice guard(ctx->device);
     hipError_t err = hipModuleLoadData(&k.module, r.code.data());
-    if (err == hipSuccess) err = hipModuleGetFunction(&k.fn, k.module, "sideaware_elementwise");
+    if (err == hipSuccess) err = hipModuleGetFunction(&k.fn, k.module, e.function_name.c_str());
     if (err != hipSuccess) {
         k.failed = true;
         k.fn = nullptr;
@@ -405,6 +421,7 @@ static int register_header(const char* header, int default_groups) {
     if (it != g_header_to_id.end()) return it->second;
     auto e = std::make_unique<KernelEntry>();
     e->header = text;
+    e->function_name = kernel_name_of(text);
     e->default_groups = default_groups > 0 ? default_groups : 0;
     g_kernels.push_back(std::move(e));
     int id = (int)g_kernels.size() - 1;
@@ -513,9 +530,12 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     // Two instantiations per op: 32-bit indices below 2 GiB, 64-bit from there on (the reference
     // also sends bases that are not 2 MiB-aligned to its 64-bit variant, sideaware.cu:1386-1388;
     // here the base only shifts the planner's b0, whatever its alignment).
-    // and, independently, one pair for arrays that fit the Infinity Cache and one for larger ones.
+    // and, independently, one pair whose input is worth keeping in the Infinity Cache and one that
+    // streams in both directions: arrays too large to be kept, and in-place launches, whose input
+    // is dead the moment it has been read.
     const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
-    const int variant = wide | (num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0);
+    const bool in_place = out0 != nullptr && out0 == in0;
+    const int variant = wide | ((in_place || num_bytes > (unsigned long long)g_tune.cache_bytes) ? 2 : 0);
 
     CompiledKernel* k = get_kernel(ctx, kernel_id, variant);
     if (!k) return;

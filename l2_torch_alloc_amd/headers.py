@@ -25,6 +25,7 @@ def _evict(flags) -> str:
 def memcpy_header() -> bytes:
     """The built-in copy (kernel id 0), spelled out: 4-byte elements, input read once."""
     return (
+        "#define KERNEL_NAME sideaware_copy_spelled_out\n"
         "typedef int o0;\ntypedef int i0;\n" + _UNUSED +
         "typedef unused o1, o2, o3, i1, i2, i3;\n"
         "constexpr bool reverse_order = false;\n" + _evict([False]) +
@@ -44,7 +45,8 @@ _ROPE_TYPES = {
 
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
                 layout: str = "qkv", backward: bool = False, unrolled: int | None = None,
-                reverse_order: bool = False, evict_input: bool = False) -> bytes:
+                reverse_order: bool = False, evict_input: bool = False,
+                stream_input: bool | None = None, stream_output: bool | None = None) -> bytes:
     """RoPE forward (or backward) in place or out of place.
 
     layout "qkv":   one tensor (B, T, n_q + 2*n_kv, head_dim); q and k heads are rotated, the
@@ -72,7 +74,13 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     rotated_heads = n_q + n_kv if layout == "qkv" else n_q
     sign_a, sign_b = ("+", "-") if backward else ("-", "+")
 
-    lines = [decl]
+    name = "sideaware_rope_%s_%s_%s_t%d_h%d_%d_d%d" % ("bwd" if backward else "fwd", dtype, layout, T, n_q,
+                                                        n_kv if layout == "qkv" else 0, head_dim)
+    lines = ["#define KERNEL_NAME %s\n" % name, decl]
+    if stream_input is not None:
+        lines.append("#define INPUT0_STREAMING %d\n" % int(stream_input))
+    if stream_output is not None:
+        lines.append("#define OUTPUT_STREAMING %d\n" % int(stream_output))
     lines.append("typedef %s o0;\ntypedef %s i0;\ntypedef float2 i1;\n" % (pair, pair))
     lines.append(_UNUSED + "typedef unused o1, o2, o3, i2, i3;\n")
     if unrolled is not None:
@@ -122,7 +130,8 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
 def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = False) -> bytes:
     """bf16 ``y = x*scale + bias``; scale and bias are two fp32 values read from the sideband
     pointer at launch, so one compiled kernel serves every (scale, bias)."""
-    lines = ["typedef __bf16 o0;\ntypedef __bf16 i0;\n", _UNUSED, "typedef unused o1, o2, o3, i1, i2, i3;\n"]
+    lines = ["#define KERNEL_NAME sideaware_scale_bias_bf16\n",
+             "typedef __bf16 o0;\ntypedef __bf16 i0;\n", _UNUSED, "typedef unused o1, o2, o3, i1, i2, i3;\n"]
     if unrolled is not None:
         lines.append("#define UNROLLED %d\n" % unrolled)
     lines.append("constexpr bool reverse_order = false;\n" + _evict([evict_input]))
@@ -149,6 +158,7 @@ def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = Fals
 def fill_header() -> bytes:
     """Writes the 32-bit sideband value to every element: an output-only op (no in0)."""
     return (
+        "#define KERNEL_NAME sideaware_fill_int32\n"
         "typedef int o0;\n" + _UNUSED + "typedef unused o1, o2, o3, i0, i1, i2, i3;\n"
         "constexpr bool reverse_order = false;\n" + _evict([]) +
         "__device__ void elementwise_op(size_t element_idx, int sideband,\n"

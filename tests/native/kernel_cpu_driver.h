@@ -31,7 +31,7 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
         for (unsigned t = 0; t < SA_WG_THREADS; t++) {
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
-            sideaware_elementwise(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val,
+            KERNEL_NAME(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val,
                                   (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
                                   p.r, p.tail_block);
         }

@@ -50,6 +50,7 @@ def ph():
     L.ph_set_trim.argtypes = [vp, sz, sz]
     L.ph_set_limit.argtypes = [vp, sz]
     L.ph_owns.restype, L.ph_owns.argtypes = ctypes.c_int, [vp, u]
+    L.ph_block_bytes.restype, L.ph_block_bytes.argtypes = sz, [vp, u]
     L.ph_stats.restype, L.ph_stats.argtypes = ctypes.c_int, [vp, ctypes.POINTER(u), ctypes.c_int]
     L.ph_backing_used.restype, L.ph_backing_used.argtypes = sz, [vp]
     L.ph_backing_live_blocks.restype, L.ph_backing_live_blocks.argtypes = sz, [vp]
@@ -135,6 +136,25 @@ def test_large_is_2mib_aligned_rounded_and_reused_lifo(pool):
     assert pool.stats()["large_hits"] == 2
     c = pool.alloc(12 * MiB)                                 # another size: no reuse
     assert c not in (a, b) and pool.stats()["large_misses"] == 3
+
+
+def test_near_fit_reuses_a_slightly_larger_region(pool):
+    a = pool.alloc(64 * MiB)
+    b = pool.alloc(72 * MiB)
+    c = pool.alloc(80 * MiB)
+    for p in (a, b, c):
+        pool.free(p)
+    # 66 MiB: no exact match; 72 MiB is within one eighth (66 + 8.25), and smaller than 80
+    got = pool.alloc(66 * MiB)
+    assert got == b and pool.L.ph_block_bytes(pool.h, got) == 72 * MiB
+    assert pool.stats()["large_hits"] == 1 and pool.stats()["bytes_live"] == 72 * MiB
+    # 40 MiB: the smallest cached region (64 MiB) is more than one eighth larger: a miss
+    misses = pool.stats()["large_misses"]
+    d = pool.alloc(40 * MiB)
+    assert d not in (a, b, c) and pool.stats()["large_misses"] == misses + 1
+    pool.free(got)
+    assert pool.stats()["bytes_cached_large"] == (64 + 72 + 80) * MiB   # goes back under its own size
+    assert pool.alloc(72 * MiB) == b
 
 
 def test_direct_entry_points_are_always_large(pool):
@@ -309,7 +329,9 @@ def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph):
                 rounded = (ph.ph_round_large(n) if n >= 8 * MiB else ph.ph_small_class_size(n))
                 assert p % (2 * MiB if n >= 8 * MiB else 512) == 0
                 assert p not in live
-                live[p] = rounded
+                held = ph.ph_block_bytes(pool.h, p)
+                assert rounded <= held <= rounded + rounded // 8      # exact, or a near fit handed out whole
+                live[p] = held
             if step % 500 == 0:
                 spans = sorted((p, p + n) for p, n in live.items())
                 assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "live blocks overlap"
