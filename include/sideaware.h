@@ -111,8 +111,8 @@ int sideaware_xcd_dealing_verified(void);
 const char* sideaware_last_error(void);
 void sideaware_clear_error(void);
 /* Compiles header + template for gfx950 without touching a device. variant bit 0: 0 = 32-bit indices
- * (arrays below 2 GiB), 1 = 64-bit indices; bit 1: 0 = out of place and the array fits the
- * Infinity Cache, 1 = in place or larger (everything streams).  Returns 0 on success; the compiler
+ * (arrays below 2 GiB), 1 = 64-bit indices; bit 1: 0 = the array fits the Infinity Cache
+ * (outputs written plainly), 1 = larger (everything streams).  Returns 0 on success; the compiler
  * log (possibly empty) is copied to `log`. */
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity);
 /* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */

@@ -31,9 +31,9 @@ static const char* kKernelTemplate =
     ;
 
 // Kernel id 0: a bit-exact copy, four bytes per element so that sixteen bytes make one vector.
-// No input is marked evict and UNROLLED is left at 1: one workgroup moves one 4 KiB chunk, the
-// source read plainly and the destination written with the streaming hint (both streaming once the
-// array no longer fits the Infinity Cache): the fastest combination measured on MI355X.
+// The source is marked evict (read once, with the streaming hint) and UNROLLED is left at 1: one
+// workgroup moves one 4 KiB chunk.  The destination is written plainly while it fits the Infinity
+// Cache, so the next kernel finds it there, and with the streaming hint beyond that.
 static const char* kMemcpyHeader = R"SA_HDR(
 #define KERNEL_NAME sideaware_copy
 typedef int o0;
@@ -42,7 +42,7 @@ struct unused {};
 typedef unused o1, o2, o3, i1, i2, i3;
 
 constexpr bool reverse_order = false;
-constexpr bool input_evict[4] = {false, false, false, false};
+constexpr bool input_evict[4] = {true, false, false, false};
 
 __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
                                                o0 &out0, o1 &out1, o2 &out2, o3 &out3,
@@ -79,7 +79,7 @@ struct Tuning {
     long long slot_run = 1;          // tiles a workgroup takes in a row; 0 = one contiguous block each
     long long one_shot = 1;          // 1: one workgroup per tile unless the caller fixes the groups
     long long cache_bytes = 256ll << 20;   // arrays larger than this are compiled to stream in both directions
-    long long nt_store = 2;          // nontemporal stores: 0 never, 1 always, 2 unless an input is marked evict
+    long long nt_store = 2;          // nontemporal stores: 0 never, 1 always, 2 only for arrays beyond the Infinity Cache
     long long groups_cap = 8;        // upper bound on default workgroups per CU
     long long wg_threads = 256;
 };
@@ -530,12 +530,10 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     // Two instantiations per op: 32-bit indices below 2 GiB, 64-bit from there on (the reference
     // also sends bases that are not 2 MiB-aligned to its 64-bit variant, sideaware.cu:1386-1388;
     // here the base only shifts the planner's b0, whatever its alignment).
-    // and, independently, one pair whose input is worth keeping in the Infinity Cache and one that
-    // streams in both directions: arrays too large to be kept, and in-place launches, whose input
-    // is dead the moment it has been read.
+    // and, independently, one pair for arrays whose result fits the Infinity Cache (written plainly,
+    // so the next kernel finds it there) and one for larger arrays (everything streams).
     const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
-    const bool in_place = out0 != nullptr && out0 == in0;
-    const int variant = wide | ((in_place || num_bytes > (unsigned long long)g_tune.cache_bytes) ? 2 : 0);
+    const int variant = wide | (num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0);
 
     CompiledKernel* k = get_kernel(ctx, kernel_id, variant);
     if (!k) return;

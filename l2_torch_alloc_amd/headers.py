@@ -28,7 +28,7 @@ def memcpy_header() -> bytes:
         "#define KERNEL_NAME sideaware_copy_spelled_out\n"
         "typedef int o0;\ntypedef int i0;\n" + _UNUSED +
         "typedef unused o1, o2, o3, i1, i2, i3;\n"
-        "constexpr bool reverse_order = false;\n" + _evict([False]) +
+        "constexpr bool reverse_order = false;\n" + _evict([True]) +
         "__device__ void elementwise_op(size_t element_idx, int sideband,\n"
         "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
         "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {\n"
@@ -45,7 +45,7 @@ _ROPE_TYPES = {
 
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
                 layout: str = "qkv", backward: bool = False, unrolled: int | None = None,
-                reverse_order: bool = False, evict_input: bool = False,
+                reverse_order: bool = False, evict_input: bool = True,
                 stream_input: bool | None = None, stream_output: bool | None = None) -> bytes:
     """RoPE forward (or backward) in place or out of place.
 
@@ -87,8 +87,7 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
         lines.append("#define UNROLLED %d\n" % unrolled)
     lines.append("constexpr bool reverse_order = %s;\n" % ("true" if reverse_order else "false"))
     # The table is re-read by every head of a token and must stay cached.  The activations are
-    # read once: either they are read with the streaming hint (evict_input) or, by default,
-    # written with it.
+    # read once, with the streaming hint.
     lines.append(_evict([evict_input, False]))
     lines.append(
         "constexpr int rope_T = %d;\n"
@@ -127,7 +126,7 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     return "".join(lines).encode()
 
 
-def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = False) -> bytes:
+def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = True) -> bytes:
     """bf16 ``y = x*scale + bias``; scale and bias are two fp32 values read from the sideband
     pointer at launch, so one compiled kernel serves every (scale, bias)."""
     lines = ["#define KERNEL_NAME sideaware_scale_bias_bf16\n",
