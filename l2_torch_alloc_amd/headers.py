@@ -154,6 +154,62 @@ def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = True
     return "".join(lines).encode()
 
 
+def mxfp8_quantize_header(unrolled: int | None = None) -> bytes:
+    """bf16 -> MXFP8 (OCP Microscaling: E4M3 elements with one E8M0 scale byte per 32 elements).
+
+    The op the reference cites as the reason for its ``vector_op`` hook and sideband pointer
+    (``sideaware.cu:81-83``): the maximum magnitude of 32 consecutive elements is needed before any
+    of them can be converted.  A 16-byte vector holds 8 bf16 elements, so a block is 4 neighbouring
+    lanes, and the maximum travels between them with two lane exchanges.  in0 = bf16 input,
+    out0 = E4M3 bytes, the sideband pointer receives the scale bytes (element count / 32 of them).
+    The element count must be a multiple of 32 so that no block is cut by the end of the array.
+
+    shared_exp = floor(log2(max|x|)) - 8, clamped to [-127, 127] (an all-zero block gets -127);
+    scale byte = shared_exp + 127; element = E4M3(x * 2^-shared_exp), round to nearest even,
+    saturated at +-448.  Finite inputs.
+    """
+    lines = ["#define KERNEL_NAME sideaware_mxfp8_quantize\n",
+             "typedef unsigned char o0;\ntypedef __bf16 i0;\n", _UNUSED,
+             "typedef unused o1, o2, o3, i1, i2, i3;\n"]
+    if unrolled is not None:
+        lines.append("#define UNROLLED %d\n" % unrolled)
+    lines.append("constexpr bool reverse_order = false;\n" + _evict([True]))
+    lines.append(
+        "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}\n"
+        "#define CUSTOM_VECTOR_OP\n"
+        "__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size,\n"
+        "                          o0 *out0, o1 *out1, o2 *out2, o3 *out3,\n"
+        "                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,\n"
+        "                          int* sideband_memory, int sideband_value) {\n"
+        "    float v[8];\n"
+        "    float amax = 0.0f;\n"
+        "    #pragma unroll\n"
+        "    for (int i = 0; i < 8; i++) { v[i] = (float)in0[i]; amax = fmaxf(amax, fabsf(v[i])); }\n"
+        "    // a block of 32 elements is 4 neighbouring lanes: lanes 4k..4k+3 of the wave\n"
+        "    amax = fmaxf(amax, __shfl_xor(amax, 1));\n"
+        "    amax = fmaxf(amax, __shfl_xor(amax, 2));\n"
+        "    // floor(log2(amax)) is the exponent field of the float (a bf16 subnormal widens to an\n"
+        "    // fp32 subnormal with field 0, far below the clamp anyway)\n"
+        "    int shared_exp = (int)((__float_as_uint(amax) >> 23) & 0xff) - 127 - 8;\n"
+        "    if (amax == 0.0f || shared_exp < -127) shared_exp = -127;\n"
+        "    if (shared_exp > 127) shared_exp = 127;\n"
+        "    if ((vec_idx & 3) == 0) ((unsigned char*)sideband_memory)[vec_idx >> 2] = (unsigned char)(shared_exp + 127);\n"
+        "    #pragma unroll\n"
+        "    for (int i = 0; i < 8; i += 2) {\n"
+        "        // two exact power-of-two steps: 2^127 and 2^-127 are not both normal floats\n"
+        "        float a = ldexpf(v[i], -shared_exp), b = ldexpf(v[i + 1], -shared_exp);\n"
+        "        a = fminf(fmaxf(a, -448.0f), 448.0f);\n"
+        "        b = fminf(fmaxf(b, -448.0f), 448.0f);\n"
+        "        const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);\n"
+        "        out0[i] = (unsigned char)(packed & 0xff);\n"
+        "        out0[i + 1] = (unsigned char)((packed >> 8) & 0xff);\n"
+        "    }\n"
+        "}\n")
+    return "".join(lines).encode()
+
+
 def fill_header() -> bytes:
     """Writes the 32-bit sideband value to every element: an output-only op (no in0)."""
     return (

@@ -104,6 +104,24 @@ def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[tor
     return out
 
 
+def mxfp8_quantize(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None):
+    """bf16 -> MXFP8: returns (E4M3 bytes as a uint8 tensor shaped like x, E8M0 scale bytes, one
+    per 32 consecutive elements).  ``x.numel()`` must be a multiple of 32."""
+    assert x.dtype == torch.bfloat16 and x.is_contiguous() and x.numel() % 32 == 0
+    if q is None:
+        q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    if scales is None:
+        scales = torch.empty(x.numel() // 32, dtype=torch.uint8, device=x.device)
+    assert q.dtype == torch.uint8 and q.numel() == x.numel() and scales.numel() == x.numel() // 32
+    kid = _kernel(("mxfp8_quantize",), headers.mxfp8_quantize_header)
+    device, stream = torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream
+    # num_bytes is the byte length of the wider array, the bf16 input, which the custom-op wrapper
+    # cannot know (it sizes the launch from out0, as the reference's does): call the C entry point.
+    wrapper.library().sideaware_elementwise(kid, x.numel() * 2, q.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
+                                            scales.data_ptr(), 0, 0, 0, device, stream)
+    return q, scales
+
+
 def fill_int32(out: torch.Tensor, value: int):
     """Writes a 32-bit pattern over ``out`` (byte size a multiple of 16): an output-only op."""
     kid = _kernel(("fill",), headers.fill_header)

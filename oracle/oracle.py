@@ -47,12 +47,19 @@ def lib() -> ctypes.CDLL:
         L.oracle_rope_forward_heads_bf16.argtypes = [vp, vp, vp, ci, ci, ci, ci]
         L.oracle_scale_bias_bf16.argtypes = [vp, vp, cf, cf, sz]
         L.oracle_memcpy.argtypes = [vp, vp, sz]
+        L.oracle_mxfp8_quantize.argtypes = [vp, vp, vp, sz]
+        L.oracle_mxfp8_dequantize.argtypes = [vp, vp, vp, sz]
+        L.oracle_f32_to_e4m3.argtypes = [cf]
+        L.oracle_f32_to_e4m3.restype = ctypes.c_uint8
+        L.oracle_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+        L.oracle_e4m3_to_f32.restype = cf
         L.oracle_validate_f32.argtypes = [vp, vp, sz, cf]
         L.oracle_validate_f32.restype = sz
         for name in ("oracle_f32_to_bf16_array", "oracle_bf16_to_f32_array", "oracle_freqs_cis",
                      "oracle_rope_forward_qkv_f32", "oracle_rope_backward_qkv_f32",
                      "oracle_rope_forward_heads_f32", "oracle_rope_backward_heads_f32",
-                     "oracle_rope_forward_heads_bf16", "oracle_scale_bias_bf16", "oracle_memcpy"):
+                     "oracle_rope_forward_heads_bf16", "oracle_scale_bias_bf16", "oracle_memcpy",
+                     "oracle_mxfp8_quantize", "oracle_mxfp8_dequantize"):
             getattr(L, name).restype = None
         _lib = L
     return _lib
@@ -148,6 +155,37 @@ def scale_bias_bf16(x_bits, scale: float, bias: float) -> np.ndarray:
     out = np.empty_like(x_bits)
     lib().oracle_scale_bias_bf16(_p(out), _p(x_bits), float(scale), float(bias), x_bits.size)
     return out
+
+
+def mxfp8_quantize(x_bits):
+    """bf16 bit patterns (count a multiple of 32) -> (E4M3 bytes, E8M0 scale bytes, one per 32)."""
+    x_bits = _u16(x_bits)
+    assert x_bits.size % 32 == 0
+    q = np.empty(x_bits.shape, dtype=np.uint8)
+    scales = np.empty(x_bits.size // 32, dtype=np.uint8)
+    lib().oracle_mxfp8_quantize(_p(q), _p(scales), _p(x_bits), x_bits.size)
+    return q, scales
+
+
+def mxfp8_dequantize(q, scales) -> np.ndarray:
+    q = np.ascontiguousarray(q, dtype=np.uint8)
+    scales = np.ascontiguousarray(scales, dtype=np.uint8)
+    assert q.size == scales.size * 32
+    out = np.empty(q.shape, dtype=np.uint16)
+    lib().oracle_mxfp8_dequantize(_p(out), _p(q), _p(scales), q.size)
+    return out
+
+
+def f32_to_e4m3(values) -> np.ndarray:
+    L = lib()
+    return np.array([L.oracle_f32_to_e4m3(float(v)) for v in np.asarray(values, dtype=np.float32).ravel()],
+                    dtype=np.uint8)
+
+
+def e4m3_to_f32(codes) -> np.ndarray:
+    L = lib()
+    return np.array([L.oracle_e4m3_to_f32(int(c)) for c in np.asarray(codes, dtype=np.uint8).ravel()],
+                    dtype=np.float32)
 
 
 def memcpy(src: np.ndarray) -> np.ndarray:

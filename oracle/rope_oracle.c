@@ -30,6 +30,11 @@
  *   oracle_f32_to_bf16      torch.Tensor.to(torch.bfloat16) on CPU, all 2^16 high
  *                           halves x several low halves, NaN/Inf included
  *   oracle_scale_bias_bf16  torch CPU fp32 multiply, add, .to(bfloat16)
+ *   oracle_f32_to_e4m3      torch.Tensor.to(torch.float8_e4m3fn) on CPU over every in-range value
+ *                           on a fine grid and every midpoint between neighbouring E4M3 values
+ *   oracle_mxfp8_quantize   closed forms (power-of-two blocks, zero block, the scale of a block
+ *                           whose maximum sits just below / at a power of two), the error bound
+ *                           of the format, and quantize(dequantize(quantize(x))) == quantize(x)
  */
 #include <math.h>
 #include <stddef.h>
@@ -238,6 +243,80 @@ void oracle_scale_bias_bf16(uint16_t *y, const uint16_t *x, float scale, float b
         float p = oracle_bf16_to_f32(x[i]) * scale;
         float r = p + bias;
         y[i] = oracle_f32_to_bf16(r);
+    }
+}
+
+/* ---- bf16 -> MXFP8 (OCP Microscaling v1.0: E4M3 elements, one E8M0 scale per 32) -------- */
+
+/* The reference names this op as the reason its template has a vector_op hook and a sideband
+ * pointer ("BF16 -> MXFP8 with microscaling where we need the absmax over 32 elements",
+ * sideaware.cu:81-83) but ships no implementation; this follows the OCP MX specification:
+ *   shared_exp = floor(log2(max|x|)) - 8        (8 = exponent of the largest E4M3 binade)
+ *   scale byte = clamp(shared_exp, -127, 127) + 127, an all-zero block gets scale byte 0
+ *   element    = E4M3( x * 2^-shared_exp ), round to nearest even, saturating at +-448
+ * Finite inputs only. */
+
+/* fp32 -> E4M3 (4 exponent bits, bias 7, 3 mantissa bits, no infinities, 0x7f/0xff = NaN),
+ * round to nearest even, saturating: |v| > 448 -> 448. */
+uint8_t oracle_f32_to_e4m3(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+    float a = fabsf(v);
+    if (a != a) return (uint8_t)(sign | 0x7f);
+    if (a >= 448.0f) return (uint8_t)(sign | 0x7e);
+    int e;
+    float m = frexpf(a, &e);                       /* a = m * 2^e, m in [0.5, 1) */
+    int exp = e - 1;                               /* a = (2m) * 2^exp, 2m in [1, 2) */
+    if (a == 0.0f || exp < -6) {                   /* zero and subnormals: quantum 2^-9 */
+        int k = (int)nearbyintf(a * 512.0f);       /* default rounding mode: nearest even; 0..8 */
+        return (uint8_t)(sign | k);                /* 8 is the encoding of the smallest normal */
+    }
+    float q = (2.0f * m) * 8.0f;                   /* in [8, 16): mantissa with 3 fraction bits */
+    int k = (int)nearbyintf(q);                    /* 8..16 */
+    if (k == 16) { k = 8; exp += 1; }
+    if (exp > 8 || (exp == 8 && k > 14)) return (uint8_t)(sign | 0x7e);
+    return (uint8_t)(sign | ((exp + 7) << 3) | (k - 8));
+}
+
+float oracle_e4m3_to_f32(uint8_t b) {
+    int sign = b & 0x80, e = (b >> 3) & 0xf, m = b & 7;
+    float v;
+    if (e == 0xf && m == 7) v = NAN;
+    else if (e == 0) v = ldexpf((float)m, -9);
+    else v = ldexpf((float)(8 + m), e - 7 - 3);
+    return sign ? -v : v;
+}
+
+/* x: n bf16 bit patterns, n a multiple of 32.  q: n E4M3 bytes.  scales: n/32 E8M0 bytes. */
+void oracle_mxfp8_quantize(uint8_t *q, uint8_t *scales, const uint16_t *x, size_t n) {
+    for (size_t b = 0; b < n / 32; b++) {
+        float amax = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            float a = fabsf(oracle_bf16_to_f32(x[b * 32 + i]));
+            if (a > amax) amax = a;
+        }
+        int shared_exp = -127;
+        if (amax > 0.0f) {
+            int e;
+            (void)frexpf(amax, &e);                /* amax = m * 2^e, m in [0.5,1): floor(log2) = e - 1 */
+            shared_exp = (e - 1) - 8;
+            if (shared_exp < -127) shared_exp = -127;
+            if (shared_exp > 127) shared_exp = 127;
+        }
+        scales[b] = (uint8_t)(shared_exp + 127);
+        for (int i = 0; i < 32; i++) {
+            float v = ldexpf(oracle_bf16_to_f32(x[b * 32 + i]), -shared_exp);
+            q[b * 32 + i] = oracle_f32_to_e4m3(v);
+        }
+    }
+}
+
+/* bf16( E4M3 element * 2^(scale - 127) ): exact, an element has 4 significant bits. */
+void oracle_mxfp8_dequantize(uint16_t *x, const uint8_t *q, const uint8_t *scales, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float v = ldexpf(oracle_e4m3_to_f32(q[i]), (int)scales[i / 32] - 127);
+        x[i] = oracle_f32_to_bf16(v);
     }
 }
 

@@ -8,6 +8,7 @@
 #include <string>
 #include <vector>
 
+#include "../../l2_torch_alloc_amd/csrc/launch_plan.h"
 #include "../../l2_torch_alloc_amd/csrc/pool.h"
 
 using namespace sideaware;
@@ -97,6 +98,14 @@ const char* ph_log(void* h) {
     return H->joined.c_str();
 }
 void ph_clear_log(void* h) { ((Harness*)h)->backing.log.clear(); }
+
+// out: full_tiles, b0, u_count, run, r, tail_block, slots, grid
+void ph_plan_launch(uint64_t base, long long num_vectors, int tile_vectors, int num_xcds, uint64_t stripe_bytes,
+                    long long slot_run, long long slots_wanted, long long* out) {
+    LaunchPlan p = plan_launch(base, num_vectors, tile_vectors, num_xcds, stripe_bytes, slot_run, slots_wanted);
+    out[0] = p.full_tiles; out[1] = p.b0; out[2] = p.u_count; out[3] = p.run;
+    out[4] = p.r; out[5] = p.tail_block; out[6] = p.slots; out[7] = p.grid;
+}
 
 size_t ph_round_large(size_t b) { return Pool::round_large(b); }
 size_t ph_small_class_size(size_t b) { return Pool::small_class_size(b); }

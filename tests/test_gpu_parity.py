@@ -255,6 +255,32 @@ def test_scale_bias_bf16_vs_oracle_and_golden(sa):
     assert_no_library_error(sa)
 
 
+def test_mxfp8_quantize_vs_oracle(sa):
+    # the vector_op + sideband op: bf16 -> E4M3 bytes + one E8M0 scale byte per 32 elements
+    from l2_torch_alloc_amd import ops
+    gen = torch.Generator().manual_seed(17)
+    n = 32 * 40000 + 32 * 7                       # many tiles and a tail
+    mag = torch.exp(torch.rand(n // 32, generator=gen) * 40 - 20).repeat_interleave(32)
+    xh = (torch.randn(n, generator=gen) * mag).to(torch.bfloat16)
+    xh[:32] = 0                                   # an all-zero block
+    xh[32:64] = 1.0                               # a power-of-two block
+    xh[64] = -1.9921875                           # saturates at -448 after scaling
+    q, s = ops.mxfp8_quantize(xh.cuda())
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    want_q, want_s = O.mxfp8_quantize(bits(xh))
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(q.cpu().numpy(), want_q)
+    # size-independent property at a large size: quantising the dequantised values changes nothing
+    big = (torch.randn(64 * MiB // 2, generator=gen) * 3).to(torch.bfloat16).cuda()
+    q1, s1 = ops.mxfp8_quantize(big)
+    deq = (q1.view(torch.float8_e4m3fn).float() *
+           torch.exp2(s1.float() - 127).repeat_interleave(32)).to(torch.bfloat16)
+    q2, s2 = ops.mxfp8_quantize(deq)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(s1, s2)
+
+
 # --------------------------------------------------------------------------------------- RoPE
 
 def rel_err(got: np.ndarray, want: np.ndarray) -> float:

@@ -209,3 +209,71 @@ def test_memcpy_and_validate():
     ref = np.array([1.0, 2.0, np.inf, 0.0], dtype=np.float32)
     got = np.array([1.0 + 5e-6, 2.1, 123.0, 2e-5], dtype=np.float32)
     assert O.validate_f32(got, ref, 1e-5) == 2      # 2.1 and 2e-5 fault; inf is skipped
+
+
+# ---------------------------------------------------------------- MXFP8 (E4M3 + E8M0 per 32)
+
+def _torch_e4m3(values: np.ndarray) -> np.ndarray:
+    t = torch.from_numpy(np.asarray(values, dtype=np.float32).copy())
+    return t.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+
+
+def test_e4m3_decode_table():
+    codes = np.arange(256, dtype=np.uint8)
+    mine = O.e4m3_to_f32(codes)
+    theirs = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    nan = np.isnan(theirs)
+    assert np.array_equal(np.isnan(mine), nan)
+    assert np.array_equal(mine[~nan], theirs[~nan])
+    assert float(np.nanmax(mine)) == 448.0
+
+
+def test_e4m3_encode_matches_torch_on_values_midpoints_and_a_fine_grid():
+    pos = np.sort(O.e4m3_to_f32(np.arange(0, 0x7f, dtype=np.uint8)))       # every finite magnitude
+    mids = (pos[:-1].astype(np.float64) + pos[1:]) / 2                       # exact ties
+    eps = np.concatenate([np.nextafter(mids.astype(np.float32), np.float32(np.inf)),
+                          np.nextafter(mids.astype(np.float32), np.float32(-np.inf))])
+    grid = rng(1).uniform(-448, 448, 20000).astype(np.float32)
+    tiny = rng(2).uniform(-0.02, 0.02, 5000).astype(np.float32)
+    vals = np.concatenate([pos, -pos, mids.astype(np.float32), -mids.astype(np.float32), eps, grid, tiny])
+    vals = vals[np.abs(vals) <= 448]
+    assert np.array_equal(O.f32_to_e4m3(vals), _torch_e4m3(vals))
+    # saturation instead of NaN beyond the largest value
+    assert O.f32_to_e4m3([449.0, 1e9, -1e9]).tolist() == [0x7e, 0x7e, 0xfe]
+
+
+def test_mxfp8_closed_forms():
+    ones = O.f32_to_bf16(np.ones(32, dtype=np.float32))
+    q, s = O.mxfp8_quantize(ones)
+    # max 1 = 2^0: shared exponent 0 - 8 = -8, scale byte 119; 1 * 2^8 = 256 = 0x78 in E4M3
+    assert s.tolist() == [119] and set(q.tolist()) == {0x78}
+    zeros = np.zeros(32, dtype=np.uint16)
+    q, s = O.mxfp8_quantize(zeros)
+    assert s.tolist() == [0] and not q.any()
+    # the largest element always lands in [256, 448]: just below a power of two it saturates
+    blk = np.full(32, 0.25, dtype=np.float32)
+    blk[5] = -1.9921875                        # bf16-exact, floor(log2) = 0 -> x * 256 = -510 -> -448
+    q, s = O.mxfp8_quantize(O.f32_to_bf16(blk))
+    assert s.tolist() == [119] and q[5] == 0xfe and q[0] == O.f32_to_e4m3([64.0])[0]
+    blk[5] = 2.0                               # at the power of two the scale steps up
+    q, s = O.mxfp8_quantize(O.f32_to_bf16(blk))
+    assert s.tolist() == [120] and q[5] == 0x78 and q[0] == O.f32_to_e4m3([32.0])[0]
+
+
+def test_mxfp8_error_bound_and_idempotence():
+    x = (rng(3).standard_normal(32 * 512) * np.exp(rng(4).uniform(-20, 20, 32 * 512))).astype(np.float32)
+    xb = O.f32_to_bf16(x)
+    q, s = O.mxfp8_quantize(xb)
+    back = O.bf16_to_f32(O.mxfp8_dequantize(q, s)).reshape(-1, 32).astype(np.float64)
+    orig = O.bf16_to_f32(xb).reshape(-1, 32).astype(np.float64)
+    scale = np.ldexp(1.0, s.astype(np.int64) - 127)[:, None]
+    # within half an E4M3 step of the element's binade (2^-4 relative), or half the smallest
+    # subnormal step of the block, or the saturation gap (448 vs < 512) for the block maximum
+    err = np.abs(back - orig)
+    bound = np.maximum(np.abs(orig) * 2.0 ** -4, scale * 2.0 ** -10)
+    sat = np.abs(orig) > 448 * scale
+    assert np.all(err[~sat] <= bound[~sat] * (1 + 1e-12))
+    assert np.all(err[sat] <= 64 * scale.repeat(32, 1)[sat])
+    # quantising the dequantised values changes nothing
+    q2, s2 = O.mxfp8_quantize(O.mxfp8_dequantize(q, s))
+    assert np.array_equal(q2, q) and np.array_equal(s2[s != 0], s[s != 0])

@@ -347,3 +347,56 @@ def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph):
         assert pool.L.ph_backing_used(pool.h) == 0 and pool.stats()["bytes_reserved"] == 0
     finally:
         pool.close()
+
+
+def test_concurrent_callers_keep_the_pool_consistent(ph):
+    # PyTorch may call the allocator from several threads (the reference has no lock at all):
+    # eight threads churn one pool; ctypes drops the GIL during each call.
+    import threading
+    pool = P(ph, capacity=32 * GiB)
+    errors = []
+    live_per_thread = [dict() for _ in range(8)]
+
+    def worker(tid):
+        rng = random.Random(100 + tid)
+        live = live_per_thread[tid]
+        try:
+            for _ in range(3000):
+                if live and rng.random() < 0.5:
+                    p = rng.choice(list(live))
+                    if pool.free(p, stream=tid) != 0:
+                        errors.append("free failed")
+                    del live[p]
+                else:
+                    n = int(4096 * 2 ** (rng.random() * 15))
+                    p = pool.alloc(n, stream=tid)
+                    if p == 0 or p in live:
+                        errors.append("bad pointer")
+                        continue
+                    live[p] = ph.ph_block_bytes(pool.h, p)
+        except Exception as e:  # pragma: no cover
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    try:
+        assert not errors, errors[:3]
+        everything = {}
+        for live in live_per_thread:
+            for p, n in live.items():
+                assert p not in everything, "one block handed to two threads"
+                everything[p] = n
+        spans = sorted((p, p + n) for p, n in everything.items())
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "live blocks overlap"
+        st = pool.stats()
+        assert st["bytes_live"] == sum(everything.values())
+        assert st["bytes_reserved"] == pool.L.ph_backing_used(pool.h)
+        for p in everything:
+            assert pool.free(p) == 0
+        pool.L.ph_release_unused(pool.h)
+        assert pool.L.ph_backing_used(pool.h) == 0
+    finally:
+        pool.close()
