@@ -104,6 +104,9 @@ int sideaware_hash_mask(void);
 /* Upper bound on the device bytes the pool may hold (0 = none): a request that would pass it is
  * answered like one the device refused (caches are given back, then null). */
 void sideaware_reserve_limit(size_t bytes);
+/* Size of the arenas that large regions are carved from (default 4 GiB); 0 gives every large
+ * region a driver allocation of its own, as in the reference. */
+void sideaware_arena_bytes(size_t bytes);
 int sideaware_num_xcds(void);
 /* 1 when the start-up probe found workgroup i of a launch on XCD i % num_xcds. */
 int sideaware_xcd_dealing_verified(void);

@@ -72,6 +72,11 @@ void* Pool::backing_acquire_locked(size_t bytes) {
     return backing_->acquire(bytes);
 }
 
+void Pool::set_arena_bytes(size_t bytes) {
+    std::lock_guard<std::mutex> g(mu_);
+    arena_bytes_ = bytes ? round_large(bytes) : 0;
+}
+
 void Pool::note_reserved(int64_t delta) {
     st_.bytes_reserved = (uint64_t)((int64_t)st_.bytes_reserved + delta);
     st_.peak_reserved = std::max(st_.peak_reserved, st_.bytes_reserved);
@@ -81,55 +86,170 @@ void Pool::note_reserved(int64_t delta) {
 // Large path
 // ---------------------------------------------------------------------------------------------
 
-// Hands cached large blocks back to the backing store until at most `down_to` bytes remain
-// cached.  Mirrors unmap_free_allocations (sideaware.cu:873-906): the device is drained first,
-// because a cached block may still be in use by work queued before it was freed.
-size_t Pool::trim_large_locked(size_t down_to) {
-    if (st_.bytes_cached_large <= down_to) return 0;
-    backing_->sync_device();
-    st_.device_syncs++;
-    size_t released = 0;
-    for (auto it = large_cache_.begin(); it != large_cache_.end() && st_.bytes_cached_large > down_to;) {
-        auto& vec = it->second;
-        // oldest first: the most recently freed blocks are the likeliest to be asked for again
-        size_t n = 0;
-        while (n < vec.size() && st_.bytes_cached_large > down_to) {
-            backing_->release(vec[n].ptr, vec[n].bytes);
-            st_.backing_releases++;
-            st_.bytes_cached_large -= vec[n].bytes;
-            note_reserved(-(int64_t)vec[n].bytes);
-            released += vec[n].bytes;
-            n++;
+namespace {
+// Tag of a free extent whose pages were last freed on more than one stream.
+void* const kMixedStreams = (void*)(uintptr_t)1;
+}  // namespace
+
+// Adds a free extent, merging it with free neighbours of the same arena.
+void Pool::extent_insert_locked(uintptr_t addr, Extent e) {
+    auto erase_size = [&](size_t bytes, uintptr_t a) {
+        auto range = free_by_size_.equal_range(bytes);
+        for (auto it = range.first; it != range.second; ++it) {
+            if (it->second == a) { free_by_size_.erase(it); return; }
         }
-        vec.erase(vec.begin(), vec.begin() + n);
-        if (vec.empty()) it = large_cache_.erase(it); else ++it;
+    };
+    auto next = free_by_addr_.lower_bound(addr);
+    if (next != free_by_addr_.end() && next->second.arena == e.arena && addr + e.bytes == next->first) {
+        if (next->second.stream != e.stream) e.stream = kMixedStreams;
+        e.bytes += next->second.bytes;
+        erase_size(next->second.bytes, next->first);
+        next = free_by_addr_.erase(next);
+    }
+    if (next != free_by_addr_.begin()) {
+        auto prev = std::prev(next);
+        if (prev->second.arena == e.arena && prev->first + prev->second.bytes == addr) {
+            if (prev->second.stream != e.stream) e.stream = kMixedStreams;
+            addr = prev->first;
+            e.bytes += prev->second.bytes;
+            erase_size(prev->second.bytes, prev->first);
+            free_by_addr_.erase(prev);
+        }
+    }
+    free_by_addr_[addr] = e;
+    free_by_size_.emplace(e.bytes, addr);
+}
+
+// Best fit from the free extents; the remainder stays free.  Pages that were freed on another
+// stream are waited for first (stream order, as for a cached region).
+void* Pool::carve_locked(size_t rounded, void* stream) {
+    auto sit = free_by_size_.lower_bound(rounded);
+    if (sit == free_by_size_.end()) return nullptr;
+    const uintptr_t addr = sit->second;
+    auto ait = free_by_addr_.find(addr);
+    Extent e = ait->second;
+    free_by_size_.erase(sit);
+    free_by_addr_.erase(ait);
+    if (e.bytes > rounded) {
+        Extent rest = e;
+        rest.bytes = e.bytes - rounded;
+        free_by_addr_[addr + rounded] = rest;
+        free_by_size_.emplace(rest.bytes, addr + rounded);
+    }
+    st_.bytes_free_arena -= rounded;
+    if (e.stream == kMixedStreams) {
+        backing_->sync_device();
+        st_.device_syncs++;
+    } else if (e.stream != stream && e.stream != nullptr) {
+        backing_->sync_stream(e.stream);
+        st_.stream_syncs++;
+    }
+    LargeBlock blk;
+    blk.ptr = (void*)addr;
+    blk.bytes = rounded;
+    blk.last_stream = stream;
+    blk.arena = e.arena;
+    large_live_.emplace(blk.ptr, blk);
+    st_.bytes_live += rounded;
+    return blk.ptr;
+}
+
+// A fresh arena from the backing store: the configured size, or just the request if that is
+// larger, or if the backing store cannot give the configured size any more.
+bool Pool::new_arena_locked(size_t min_bytes) {
+    size_t want = std::max(arena_bytes_, min_bytes);
+    void* p = backing_acquire_locked(want);
+    if (!p && want > min_bytes) {
+        want = min_bytes;
+        p = backing_acquire_locked(want);
+    }
+    if (!p) return false;
+    assert(((uintptr_t)p % kRegionAlign) == 0);
+    note_reserved((int64_t)want);
+    st_.arenas_acquired++;
+    auto arena = std::make_unique<Arena>();
+    arena->base = (char*)p;
+    arena->bytes = want;
+    Extent e;
+    e.bytes = want;
+    e.arena = arena.get();
+    e.stream = nullptr;            // never used: nothing to wait for
+    st_.bytes_free_arena += want;
+    extent_insert_locked((uintptr_t)p, e);
+    arenas_.push_back(std::move(arena));
+    return true;
+}
+
+// Folds every cached region back into its arena's free extents.
+void Pool::flush_cache_locked() {
+    for (auto& kv : large_cache_) {
+        for (LargeBlock& blk : kv.second) {
+            Extent e;
+            e.bytes = blk.bytes;
+            e.arena = blk.arena;
+            e.stream = blk.last_stream;
+            st_.bytes_free_arena += blk.bytes;
+            extent_insert_locked((uintptr_t)blk.ptr, e);
+        }
+    }
+    large_cache_.clear();
+    st_.bytes_cached_large = 0;
+}
+
+// Returns wholly free arenas to the backing store until at most `down_to` free bytes remain in
+// arenas.  The device is drained first (unmap_free_allocations does the same,
+// sideaware.cu:873-906): freed pages may still be in use by work queued before the free.
+size_t Pool::release_free_arenas_locked(size_t down_to) {
+    size_t released = 0;
+    bool synced = false;
+    for (auto it = arenas_.begin(); it != arenas_.end() && st_.bytes_free_arena > down_to;) {
+        Arena* a = it->get();
+        auto fit = free_by_addr_.find((uintptr_t)a->base);
+        if (fit == free_by_addr_.end() || fit->second.bytes != a->bytes) { ++it; continue; }
+        if (!synced) {
+            backing_->sync_device();
+            st_.device_syncs++;
+            synced = true;
+        }
+        auto range = free_by_size_.equal_range(a->bytes);
+        for (auto sit = range.first; sit != range.second; ++sit) {
+            if (sit->second == (uintptr_t)a->base) { free_by_size_.erase(sit); break; }
+        }
+        free_by_addr_.erase(fit);
+        backing_->release(a->base, a->bytes);
+        st_.backing_releases++;
+        st_.bytes_free_arena -= a->bytes;
+        note_reserved(-(int64_t)a->bytes);
+        released += a->bytes;
+        it = arenas_.erase(it);
     }
     return released;
 }
 
-void* Pool::acquire_large_locked(size_t rounded, void* stream) {
-    void* p = backing_acquire_locked(rounded);
-    if (!p) return nullptr;
-    assert(((uintptr_t)p % kRegionAlign) == 0);
-    note_reserved((int64_t)rounded);
-    LargeBlock blk;
-    blk.ptr = p;
-    blk.bytes = rounded;
-    blk.last_stream = stream;
-    large_live_.emplace(p, blk);
-    st_.bytes_live += rounded;
-    return p;
+// Brings cached + free large bytes down to `down_to` (as far as whole arenas allow).
+size_t Pool::trim_large_locked(size_t down_to) {
+    if (st_.bytes_cached_large + st_.bytes_free_arena <= down_to) return 0;
+    flush_cache_locked();
+    return release_free_arenas_locked(down_to);
 }
 
 void* Pool::allocate_large_locked(size_t bytes, void* stream) {
     const size_t rounded = round_large(bytes);
 
-    // 1) exact-size reuse, newest first (sideaware.cu:1199-1219); failing that, the smallest
-    //    cached region that is at most one eighth larger, handed out whole.  Any 2 MiB-aligned
-    //    region serves, and a driver allocation costs hundreds of microseconds.
-    auto it = large_cache_.lower_bound(rounded);
-    while (it != large_cache_.end() && it->second.empty()) ++it;
-    if (it != large_cache_.end() && it->first <= rounded + rounded / 8) {
+    // 1) exact-size reuse, newest first (sideaware.cu:1199-1219)
+    auto it = large_cache_.find(rounded);
+    if (it == large_cache_.end() || it->second.empty()) {
+        // 2) best fit from the arenas' free extents: no waste, no driver call
+        if (void* p = carve_locked(rounded, stream)) {
+            st_.large_carves++;
+            return p;
+        }
+        // 3) the smallest cached region at most one eighth larger, handed out whole
+        it = large_cache_.lower_bound(rounded);
+        while (it != large_cache_.end() && it->second.empty()) ++it;
+        if (it != large_cache_.end() && it->first > rounded + rounded / 8) it = large_cache_.end();
+    }
+    if (it != large_cache_.end() && !it->second.empty()) {
         LargeBlock blk = it->second.back();
         it->second.pop_back();
         if (it->second.empty()) large_cache_.erase(it);
@@ -146,22 +266,28 @@ void* Pool::allocate_large_locked(size_t bytes, void* stream) {
     }
     st_.large_misses++;
 
-    // 2) trim the cache if it has outgrown its budget, then ask the backing store
-    if (st_.bytes_cached_large > trim_start_) {
+    // 4) a miss.  If cached + free bytes have outgrown their budget, fold the cache into the
+    //    arenas and give wholly free arenas back (the reference's threshold trim,
+    //    sideaware.cu:1242); what stays free may now fit the request.
+    if (st_.bytes_cached_large + st_.bytes_free_arena > trim_start_) {
         trim_large_locked(trim_end_);
         st_.trims++;
+        if (void* p = carve_locked(rounded, stream)) return p;
     }
-    if (void* p = acquire_large_locked(rounded, stream)) return p;
+    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
 
-    // 3) give back every cached large block and retry
+    // 5) the backing store refused: fold the cache back, carve if that made room, else give every
+    //    free arena back and retry
     st_.ladder_retries++;
-    trim_large_locked(0);
-    if (void* p = acquire_large_locked(rounded, stream)) return p;
+    flush_cache_locked();
+    if (void* p = carve_locked(rounded, stream)) return p;
+    release_free_arenas_locked(0);
+    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
 
-    // 4) give back empty slabs too and retry one last time
+    // 6) give back empty slabs too and retry one last time
     st_.ladder_retries++;
     release_empty_slabs_locked();
-    if (void* p = acquire_large_locked(rounded, stream)) return p;
+    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
 
     st_.failures++;
     return nullptr;

@@ -10,10 +10,14 @@
 // regions falls in the same XCD's stripe.  The pool delivers that, plus the reference's
 // caching behaviour:
 //
-//   large  (size >= threshold): dedicated region, size rounded up to 2 MiB, exact-size LIFO
-//          reuse cache (then the smallest cached region at most 1/8 larger, handed out whole),
-//          trimmed back to the backing store when it outgrows the thresholds, and the
-//          reference's four-step out-of-memory ladder (sideaware.cu:1233-1252);
+//   large  (size >= threshold): a 2 MiB-aligned region, size rounded up to 2 MiB.  Freed regions
+//          go to an exact-size LIFO reuse cache, as in the reference.  A size that is not cached
+//          is carved, best fit, from the free extents of multi-GiB arenas (a driver allocation
+//          costs hundreds of microseconds; a carve costs one), or served by a cached region at
+//          most 1/8 larger, handed out whole.  When cached plus free bytes outgrow the
+//          thresholds the cache is folded back into the arenas and wholly free arenas return to
+//          the backing store; the reference's four-step out-of-memory ladder ends in null
+//          (sideaware.cu:1233-1252);
 //   small  (size <  threshold): 512 B-granular size classes carved from slabs, so the common
 //          small request never reaches the driver (the reference forwards these to
 //          cudaMallocAsync, sideaware.cu:1326-1339).
@@ -36,6 +40,7 @@ namespace sideaware {
 constexpr size_t kRegionAlign = 2ull << 20;      // alignment and rounding of large regions
 constexpr size_t kSmallGranule = 512;            // alignment and minimum size of small blocks
 constexpr size_t kMaxSlabBytes = 64ull << 20;
+constexpr size_t kDefaultArenaBytes = 4ull << 30;
 
 // Where the bytes come from.  The HIP implementation lives in hip_backing.cpp.
 class Backing {
@@ -71,6 +76,9 @@ struct PoolStats {
     uint64_t bytes_cached_small = 0;
     uint64_t bytes_reserved = 0;    // everything held from the backing store
     uint64_t peak_reserved = 0;
+    uint64_t large_carves = 0;      // large requests carved from an arena's free extents
+    uint64_t arenas_acquired = 0;
+    uint64_t bytes_free_arena = 0;  // free extents inside arenas
 };
 constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
 
@@ -86,6 +94,9 @@ public:
     // Upper bound on bytes held from the backing store (0 = none).  A request that would pass it
     // walks the same ladder as one the device refused.
     void set_reserve_limit(size_t bytes);
+    // Size of the arenas large regions are carved from; 0 gives every region a backing
+    // allocation of its own.
+    void set_arena_bytes(size_t bytes);
 
     // always_large: the reference's direct C entry points (sideaware_malloc and friends,
     // sideaware.cu:1280-1305) never take the small path.
@@ -107,10 +118,20 @@ public:
     static int small_class_index(size_t bytes);
 
 private:
+    struct Arena {
+        char* base = nullptr;
+        size_t bytes = 0;
+    };
     struct LargeBlock {
         void* ptr = nullptr;
         size_t bytes = 0;          // rounded
         void* last_stream = nullptr;
+        Arena* arena = nullptr;
+    };
+    struct Extent {                // a free run of pages inside an arena
+        size_t bytes = 0;
+        Arena* arena = nullptr;
+        void* stream = nullptr;    // the stream its memory was last freed on, or kMixedStreams
     };
     struct Slab {
         char* base = nullptr;
@@ -133,7 +154,11 @@ private:
 
     void* allocate_large_locked(size_t bytes, void* stream);
     void* allocate_small_locked(size_t bytes, void* stream);
-    void* acquire_large_locked(size_t rounded, void* stream);
+    void* carve_locked(size_t rounded, void* stream);
+    void extent_insert_locked(uintptr_t addr, Extent e);
+    bool new_arena_locked(size_t min_bytes);
+    void flush_cache_locked();
+    size_t release_free_arenas_locked(size_t down_to);
     Slab* new_slab_locked(size_t block);
     size_t trim_large_locked(size_t down_to);
     size_t release_empty_slabs_locked();
@@ -146,9 +171,13 @@ private:
     size_t trim_start_ = 16ull << 30;
     size_t trim_end_ = 2ull << 30;
     size_t reserve_limit_ = 0;
+    size_t arena_bytes_ = kDefaultArenaBytes;
 
     std::map<size_t, std::vector<LargeBlock>> large_cache_;            // rounded size -> LIFO, sizes ordered
     std::unordered_map<void*, LargeBlock> large_live_;
+    std::vector<std::unique_ptr<Arena>> arenas_;
+    std::map<uintptr_t, Extent> free_by_addr_;
+    std::multimap<size_t, uintptr_t> free_by_size_;
     std::vector<SmallClass> small_;                                    // class index -> state
     std::unordered_map<uintptr_t, Slab*> slab_by_page_;                // addr >> 21 -> slab
     std::vector<std::unique_ptr<Slab>> slab_store_;

@@ -184,12 +184,15 @@ static size_t g_pending_trim[2] = {0, 0};
 static bool g_have_pending_trim = false;
 static size_t g_pending_limit = 0;
 static bool g_have_pending_limit = false;
+static size_t g_pending_arena = 0;
+static bool g_have_pending_arena = false;
 
 static void apply_config(Pool* pool) {
     std::lock_guard<std::mutex> g(g_config_mu);
     if (g_have_pending_threshold) pool->set_large_threshold(g_pending_threshold);
     if (g_have_pending_trim) pool->set_trim_thresholds(g_pending_trim[0], g_pending_trim[1]);
     if (g_have_pending_limit) pool->set_reserve_limit(g_pending_limit);
+    if (g_have_pending_arena) pool->set_arena_bytes(g_pending_arena);
 }
 
 void DeviceContext::initialize() {
@@ -646,6 +649,15 @@ void sideaware_reserve_limit(size_t bytes) {
         std::lock_guard<std::mutex> g(g_config_mu);
         g_pending_limit = bytes;
         g_have_pending_limit = true;
+    }
+    for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
+}
+
+void sideaware_arena_bytes(size_t bytes) {
+    {
+        std::lock_guard<std::mutex> g(g_config_mu);
+        g_pending_arena = bytes;
+        g_have_pending_arena = true;
     }
     for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
 }

@@ -64,6 +64,7 @@ _SIGNATURES = {
     "sideaware_min_sm_per_side": (_ci, []),
     "sideaware_hash_mask": (_ci, []),
     "sideaware_reserve_limit": (None, [_sz]),
+    "sideaware_arena_bytes": (None, [_sz]),
     "sideaware_num_xcds": (_ci, []),
     "sideaware_xcd_dealing_verified": (_ci, []),
     "sideaware_last_error": (ctypes.c_char_p, []),
@@ -84,7 +85,7 @@ POOL_STAT_FIELDS = (
     "large_hits", "large_misses", "small_hits", "small_carves", "slabs_acquired", "backing_acquires",
     "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
     "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
-    "peak_reserved",
+    "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena",
 )
 
 

@@ -77,6 +77,7 @@ int ph_free(void* h, uintptr_t ptr, uintptr_t stream) {
 }
 size_t ph_release_unused(void* h) { return ((Harness*)h)->pool.release_unused(); }
 void ph_set_threshold(void* h, size_t t) { ((Harness*)h)->pool.set_large_threshold(t); }
+void ph_set_arena(void* h, size_t b) { ((Harness*)h)->pool.set_arena_bytes(b); }
 void ph_set_limit(void* h, size_t b) { ((Harness*)h)->pool.set_reserve_limit(b); }
 void ph_set_trim(void* h, size_t a, size_t b) { ((Harness*)h)->pool.set_trim_thresholds(a, b); }
 size_t ph_block_bytes(void* h, uintptr_t p) { return ((Harness*)h)->pool.block_bytes((void*)p); }

@@ -64,11 +64,15 @@ def test_release_unused_gives_memory_back(sa):
     x = torch.empty(64 * MiB, dtype=torch.uint8, device="cuda")
     del x
     torch.cuda.synchronize()
-    cached = sa.sideaware_alloc_stats()["bytes_cached_large"]
-    assert cached >= 64 * MiB
+    before = sa.sideaware_alloc_stats()
+    assert before["bytes_cached_large"] >= 64 * MiB
     freed = lib.sideaware_release_unused()
-    assert freed >= cached
-    assert sa.sideaware_alloc_stats()["bytes_cached_large"] == 0
+    after = sa.sideaware_alloc_stats()
+    # the cache is folded back into the arenas and every wholly free arena returns to the driver;
+    # an arena that still holds a live region stays
+    assert after["bytes_cached_large"] == 0
+    assert after["bytes_reserved"] == before["bytes_reserved"] - freed
+    assert after["bytes_free_arena"] + after["bytes_live"] + after["bytes_cached_small"] <= after["bytes_reserved"]
 
 
 def test_out_of_memory_is_a_null_pointer_not_a_crash(sa):
@@ -96,22 +100,38 @@ def test_out_of_memory_is_a_null_pointer_not_a_crash(sa):
 def test_reserve_limit_acts_like_a_full_device(sa):
     lib = sa.library()
     lib.sideaware_release_unused()
-    held = sa.sideaware_alloc_stats()["bytes_reserved"]
-    lib.sideaware_reserve_limit(held + 256 * MiB)
+    st = sa.sideaware_alloc_stats()
+    lib.sideaware_reserve_limit(st["bytes_reserved"] + 256 * MiB)
     try:
-        ok = lib.sideaware_malloc_auto(128 * MiB, 0, None)
+        ok = lib.sideaware_malloc_auto(128 * MiB, 0, None)            # free arena space, or a small new arena
         assert ok and ok % (2 * MiB) == 0
-        assert lib.sideaware_malloc_auto(512 * MiB, 0, None) is None
+        too_much = sa.sideaware_alloc_stats()["bytes_free_arena"] + (1 << 30)
+        assert lib.sideaware_malloc_auto(too_much, 0, None) is None    # would need > 256 MiB more from the driver
+        assert sa.sideaware_alloc_stats()["failures"] == st["failures"] + 1
         lib.sideaware_free_auto(ok, 128 * MiB, 0, None)
-        # with the cached 128 MiB given back by the ladder, 200 MiB fits under the limit
-        again = lib.sideaware_malloc_auto(200 * MiB, 0, None)
-        assert again
-        lib.sideaware_free_auto(again, 200 * MiB, 0, None)
     finally:
         lib.sideaware_reserve_limit(0)
         lib.sideaware_clear_error()
     z = torch.empty(512 * MiB, dtype=torch.uint8, device="cuda")
     assert z.data_ptr() % (2 * MiB) == 0
+
+
+def test_regions_are_carved_from_arenas(sa):
+    lib = sa.library()
+    lib.sideaware_release_unused()
+    before = sa.sideaware_alloc_stats()
+    tensors = [torch.empty((24 + 2 * i) * MiB, dtype=torch.uint8, device="cuda") for i in range(8)]
+    after = sa.sideaware_alloc_stats()
+    assert all(t.data_ptr() % (2 * MiB) == 0 for t in tensors)
+    # eight different sizes, at most one new arena from the driver
+    assert after["backing_acquires"] - before["backing_acquires"] <= 1
+    assert after["large_carves"] - before["large_carves"] >= 7
+    spans = sorted((t.data_ptr(), t.data_ptr() + t.numel()) for t in tensors)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+    for i, t in enumerate(tensors):
+        t.fill_(i + 1)
+    torch.cuda.synchronize()
+    assert [int(t[0]) for t in tensors] == list(range(1, 9)) and [int(t[-1]) for t in tensors] == list(range(1, 9))
 
 
 def test_threshold_and_trim_settings_apply(sa):
@@ -120,11 +140,12 @@ def test_threshold_and_trim_settings_apply(sa):
     try:
         blocks = [torch.empty((10 + 2 * i) * MiB, dtype=torch.uint8, device="cuda") for i in range(6)]
         del blocks
-        assert sa.sideaware_alloc_stats()["bytes_cached_large"] >= 90 * MiB
-        trims = sa.sideaware_alloc_stats()["trims"]
-        z = torch.empty(50 * MiB, dtype=torch.uint8, device="cuda")     # a miss, cache over budget
         st = sa.sideaware_alloc_stats()
-        assert st["trims"] == trims + 1 and st["bytes_cached_large"] == 0
+        assert st["bytes_cached_large"] >= 90 * MiB
+        # a request no cached region and no free extent can serve: a miss with the cache over budget
+        z = torch.empty(st["bytes_free_arena"] + 64 * MiB, dtype=torch.uint8, device="cuda")
+        after = sa.sideaware_alloc_stats()
+        assert after["trims"] == st["trims"] + 1 and after["bytes_cached_large"] == 0
         del z
     finally:
         lib.sideaware_free_mapped_thresholds(16 << 30, 2 << 30)

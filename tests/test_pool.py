@@ -26,7 +26,7 @@ GiB = 1 << 30
 FIELDS = ("large_hits", "large_misses", "small_hits", "small_carves", "slabs_acquired", "backing_acquires",
           "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
           "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
-          "peak_reserved")
+          "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena")
 
 
 def build_harness():
@@ -49,6 +49,7 @@ def ph():
     L.ph_set_threshold.argtypes = [vp, sz]
     L.ph_set_trim.argtypes = [vp, sz, sz]
     L.ph_set_limit.argtypes = [vp, sz]
+    L.ph_set_arena.argtypes = [vp, sz]
     L.ph_owns.restype, L.ph_owns.argtypes = ctypes.c_int, [vp, u]
     L.ph_block_bytes.restype, L.ph_block_bytes.argtypes = sz, [vp, u]
     L.ph_stats.restype, L.ph_stats.argtypes = ctypes.c_int, [vp, ctypes.POINTER(u), ctypes.c_int]
@@ -65,8 +66,11 @@ def ph():
 
 
 class P:
-    def __init__(self, L, capacity=64 * GiB):
+    def __init__(self, L, capacity=64 * GiB, arena=0):
+        # arena=0: every large region is its own backing allocation (the reference's shape, and
+        # what the policy tests below reason about); the arena tests pass a size.
         self.L, self.h = L, L.ph_create(capacity)
+        L.ph_set_arena(self.h, arena)
 
     def close(self):
         self.L.ph_destroy(self.h)
@@ -268,6 +272,91 @@ def test_release_unused_returns_everything_cached(pool):
     assert again and pool.L.ph_owns(pool.h, again)
 
 
+# ------------------------------------------------------------------------------ arenas
+
+def test_regions_are_carved_from_one_arena_and_coalesce(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        a, b, c = pool.alloc(16 * MiB), pool.alloc(16 * MiB), pool.alloc(16 * MiB)
+        assert pool.log() == ["acquire %d" % (64 * MiB)]               # one driver call for all three
+        assert b == a + 16 * MiB and c == b + 16 * MiB
+        assert all(p % (2 * MiB) == 0 for p in (a, b, c))
+        st = pool.stats()
+        # the first request needed the driver (a miss); the next two were carved from what it brought
+        assert st["large_misses"] == 1 and st["large_carves"] == 2
+        assert st["arenas_acquired"] == 1 and st["bytes_free_arena"] == 16 * MiB
+        # a size that is not cached is carved from the arena's free tail, not from the driver
+        pool.free(b)
+        d = pool.alloc(10 * MiB)
+        assert d == c + 16 * MiB and pool.stats()["backing_acquires"] == 1
+        # the freed 16 MiB comes back exactly (LIFO cache), not through a carve
+        assert pool.alloc(16 * MiB) == b and pool.stats()["large_hits"] == 1
+        # everything freed and folded back: the extents merge into the whole arena, which goes home
+        for p in (a, b, c, d):
+            pool.free(p)
+        assert pool.L.ph_release_unused(pool.h) == 64 * MiB
+        assert pool.L.ph_backing_used(pool.h) == 0 and pool.stats()["bytes_free_arena"] == 0
+        assert "release %d" % (64 * MiB) in pool.log()
+    finally:
+        pool.close()
+
+
+def test_request_larger_than_an_arena_gets_its_own(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        p = pool.alloc(200 * MiB)
+        assert p and pool.log() == ["acquire %d" % (200 * MiB)]
+    finally:
+        pool.close()
+
+
+def test_arena_falls_back_to_the_request_size_when_memory_is_short(ph):
+    pool = P(ph, capacity=100 * MiB, arena=64 * MiB)
+    try:
+        a = pool.alloc(40 * MiB)                      # arena 1: 64 MiB
+        b = pool.alloc(30 * MiB)                      # does not fit the 24 MiB left; 64 MiB more would pass 100
+        assert a and b
+        assert pool.log() == ["acquire %d" % (64 * MiB), "acquire_failed %d" % (64 * MiB), "acquire %d" % (30 * MiB)]
+    finally:
+        pool.close()
+
+
+def test_trim_folds_the_cache_back_and_releases_whole_arenas(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        pool.L.ph_set_trim(pool.h, 100 * MiB, 0)
+        blocks = [pool.alloc(32 * MiB) for _ in range(6)]         # three arenas
+        keep = blocks[0]
+        for b in blocks[1:]:
+            pool.free(b)
+        assert pool.stats()["bytes_cached_large"] == 160 * MiB
+        pool.clear_log()
+        big = pool.alloc(48 * MiB)                                # a miss with 160 MiB cached > 100 MiB
+        assert big
+        st = pool.stats()
+        assert st["trims"] == 1 and st["bytes_cached_large"] == 0
+        log = pool.log()
+        assert log[0] == "sync_device" and log.count("release %d" % (64 * MiB)) == 2   # two wholly free arenas
+        assert pool.L.ph_owns(pool.h, keep)                       # the arena with a live region stays
+    finally:
+        pool.close()
+
+
+def test_carved_pages_wait_for_the_stream_that_freed_them(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        a = pool.alloc(32 * MiB, stream=7)
+        b = pool.alloc(32 * MiB, stream=8)
+        pool.free(a, stream=7)
+        pool.free(b, stream=8)
+        pool.L.ph_set_trim(pool.h, 0, 64 * MiB)                   # every miss folds the cache back, nothing released
+        pool.clear_log()
+        c = pool.alloc(20 * MiB, stream=7)                        # carved from pages freed on 7 and 8: mixed
+        assert c and "sync_device" in pool.log()
+    finally:
+        pool.close()
+
+
 # ------------------------------------------------------------------------------ small path
 
 def test_small_blocks_are_pooled_and_512_aligned(pool):
@@ -311,8 +400,9 @@ def test_free_null_and_foreign(pool):
 
 # ------------------------------------------------------------------------------ churn invariants
 
-def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph):
-    pool = P(ph, capacity=8 * GiB)
+@pytest.mark.parametrize("arena", [0, 256 * MiB, 4 * GiB])
+def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph, arena):
+    pool = P(ph, capacity=16 * GiB, arena=arena)
     rng = random.Random(4)
     live = {}                                         # ptr -> rounded size
     try:
@@ -338,7 +428,8 @@ def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph):
                 st = pool.stats()
                 assert st["bytes_live"] == sum(live.values())
                 assert st["bytes_reserved"] == pool.L.ph_backing_used(pool.h)
-                assert st["bytes_live"] + st["bytes_cached_large"] + st["bytes_cached_small"] <= st["bytes_reserved"]
+                assert (st["bytes_live"] + st["bytes_cached_large"] + st["bytes_cached_small"]
+                        + st["bytes_free_arena"]) <= st["bytes_reserved"]
         for p in list(live):
             assert pool.free(p) == 0
         st = pool.stats()
@@ -353,7 +444,7 @@ def test_concurrent_callers_keep_the_pool_consistent(ph):
     # PyTorch may call the allocator from several threads (the reference has no lock at all):
     # eight threads churn one pool; ctypes drops the GIL during each call.
     import threading
-    pool = P(ph, capacity=32 * GiB)
+    pool = P(ph, capacity=32 * GiB, arena=1 * GiB)
     errors = []
     live_per_thread = [dict() for _ in range(8)]
 
