@@ -44,7 +44,7 @@ _ROPE_TYPES = {
 
 
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
-                layout: str = "qkv", backward: bool = False, unrolled: int | None = None,
+                layout: str = "qkv", backward: bool = False, unrolled: int | None = 2,
                 reverse_order: bool = False, evict_input: bool = True,
                 stream_input: bool | None = None, stream_output: bool | None = None) -> bytes:
     """RoPE forward (or backward) in place or out of place.

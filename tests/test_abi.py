@@ -179,3 +179,42 @@ def test_reference_rope_header_compiles_unchanged(lib, variant):
     with open(os.path.join(REFERENCE_DIR, "kernel_rope.cuh"), "rb") as f:
         rc, log = compile_ok(lib, f.read(), variant)
     assert rc == 0, log
+
+
+def _isa_of(lib, tmp_path, header, variant):
+    """Compiles header + template for gfx950 and returns the disassembly the library wrote."""
+    dump = tmp_path / ("isa_%d.txt" % variant)
+    lib.sideaware_write_sass(str(dump).encode())
+    try:
+        rc, log = compile_ok(lib, header, variant)
+        assert rc == 0, log
+    finally:
+        lib.sideaware_write_sass(b"")
+    return dump.read_text()
+
+
+def _memory_ops(isa, kernel):
+    body = isa[isa.index("<%s>:" % kernel):]
+    body = body[:body.index("s_endpgm")]
+    loads = [l.strip() for l in body.splitlines() if "global_load_dwordx4" in l]
+    stores = [l.strip() for l in body.splitlines() if "global_store_dwordx4" in l]
+    return loads, stores
+
+
+def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
+    # the built-in copy: 16-byte loads and stores; the source is marked evict
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 0), "sideaware_copy")
+    assert loads and stores
+    assert all(" nt" in l for l in loads), loads            # read once: nontemporal
+    assert not any(" nt" in s for s in stores), stores        # fits the Infinity Cache: kept for the consumer
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 2), "sideaware_copy")
+    assert all(" nt" in l for l in loads) and all(" nt" in s for s in stores)   # larger: everything streams
+    # RoPE: the activations stream, the gathered table never does
+    rope = headers.rope_header(4096, 32, 0, 128, "bf16", "heads", unrolled=1)
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, rope, 2),
+                                "sideaware_rope_fwd_bf16_heads_t4096_h32_0_d128")
+    assert sum(" nt" in l for l in loads) == 2 and sum(" nt" not in l for l in loads) == 4, loads
+    assert all(" nt" in s for s in stores)
+    # bf16 is narrowed by the hardware's round-to-nearest-even convert, fp32 math is not fused
+    isa = _isa_of(lib, tmp_path, rope, 0)
+    assert "v_cvt_pk_bf16_f32" in isa and "v_fma_f32" not in isa and "v_pk_mul_f32" not in isa

@@ -121,6 +121,55 @@ def test_memcpy_nan_payloads_survive(sa):
     assert np.array_equal(bits(dst), bits(src))
 
 
+def test_memcpy_between_the_cache_size_and_2_gib(sa):
+    # 320 MiB + a tail: the all-streaming kernel class with 32-bit indices
+    n = 320 * MiB + 4096 + 48
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    src.random_(0, 256)
+    dst = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    assert_no_library_error(sa)
+
+
+def test_launches_replay_from_a_hip_graph(sa):
+    # a launch allocates nothing and synchronises nothing, so it can be captured; the kernels are
+    # compiled by a first eager call, outside the capture
+    from l2_torch_alloc_amd import ops
+    n = 8 * MiB + 4096
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    mid = torch.zeros_like(src)
+    dst = torch.zeros_like(src)
+    x = torch.randn(1, 64, 8, 128).to(torch.bfloat16).cuda()
+    freqs = ops.freqs_cis_table(128, 64, 500000.0).cuda()
+    x0 = x.clone()
+    torch.ops.sideaware.memcpy(mid, src)
+    ops.rope_forward_heads(x.clone(), freqs)
+    torch.cuda.synchronize()
+    eager = ops.rope_forward_heads(x0.clone(), freqs).clone()
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            torch.ops.sideaware.memcpy(mid, src)
+            torch.ops.sideaware.memcpy(dst, mid)
+            ops.rope_forward_heads(x, freqs)
+    torch.cuda.current_stream().wait_stream(side)
+    for trial in range(4):
+        src.random_(0, 256)
+        dst.zero_()
+        x.copy_(x0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src), trial
+        assert torch.equal(x, eager), trial
+    assert_no_library_error(sa)
+
+
 def test_memcpy_needs_64_bit_indices(sa):
     # 2 GiB + 64 KiB + 16 B: past the 32-bit path of the launcher (sideaware.cu:1387) and with a tail
     n = (2 << 30) + 65536 + 16
