@@ -2,6 +2,7 @@
 // Declarations and the reference interface each entry point replaces: include/sideaware.h.
 #include <hip/hip_runtime.h>
 
+#include <array>
 #include <atomic>
 #include <cctype>
 #include <cstdarg>
@@ -287,6 +288,8 @@ static DeviceContext* get_context(int device = -1) {
 // Kernel registry: header text -> id, and per (id, device, variant) the compiled function
 // ---------------------------------------------------------------------------------------------
 
+constexpr int kMaxDevices = 16;
+
 struct CompiledKernel {
     hipModule_t module = nullptr;
     hipFunction_t fn = nullptr;
@@ -302,7 +305,9 @@ struct KernelEntry {
     std::string header;
     std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`
     int default_groups = 0;     // 0: decide from occupancy
-    std::vector<CompiledKernel> compiled;   // [device * 4 + variant]; variant = 2*beyond_cache + wide_index
+    // [device * 4 + variant]; variant = 2*beyond_cache + wide_index.  Fixed size: launches keep
+    // pointers into it while other threads compile other variants.
+    std::array<CompiledKernel, kMaxDevices * 4> compiled;
 };
 
 static std::mutex g_kernels_mu;
@@ -358,9 +363,11 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
         return nullptr;
     }
     KernelEntry& e = *g_kernels[kernel_id];
-    size_t slot = (size_t)ctx->device * 4 + (size_t)(variant & 3);
-    if (e.compiled.size() <= slot) e.compiled.resize(slot + 1);
-    CompiledKernel& k = e.compiled[slot];
+    if (ctx->device >= kMaxDevices) {
+        set_error("device %d is beyond the %d devices this build keeps kernels for", ctx->device, kMaxDevices);
+        return nullptr;
+    }
+    CompiledKernel& k = e.compiled[(size_t)ctx->device * 4 + (size_t)(variant & 3)];
     unsigned gen = g_tune_generation.load();
     if (k.generation != gen) {
         if (k.module) (void)hipModuleUnload(k.module);
@@ -530,11 +537,11 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         return;
     }
 
-    // Two instantiations per op: 32-bit indices below 2 GiB, 64-bit from there on (the reference
-    // also sends bases that are not 2 MiB-aligned to its 64-bit variant, sideaware.cu:1386-1388;
-    // here the base only shifts the planner's b0, whatever its alignment).
-    // and, independently, one pair for arrays whose result fits the Infinity Cache (written plainly,
-    // so the next kernel finds it there) and one for larger arrays (everything streams).
+    // Four instantiations per op.  Index width: 32-bit below 2 GiB, 64-bit from there on (the
+    // reference also sends bases that are not 2 MiB-aligned to its 64-bit variant,
+    // sideaware.cu:1386-1388; here the base only shifts the planner's b0, whatever its alignment).
+    // Cache class: arrays whose result fits the Infinity Cache (written plainly, so the next kernel
+    // finds it there) and larger ones (everything streams).
     const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
     const int variant = wide | (num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0);
 
