@@ -30,13 +30,14 @@ MiB = 1 << 20
 GiB = 1 << 30
 HBM_PEAK_GBPS = 8000.0
 
-# HBM-side bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE in one run, WRITE_SIZE in
-# another, KiB per dispatch), each scaled by what the same counter reads for the runtime's own
-# 256 MiB buffer copy in the same run (FETCH_SIZE reads 131083.5 KiB for 262144 KiB fetched, so
-# x1.99982; WRITE_SIZE reads 262144.0, so x1.0).  Source: profiles/*_hbm_traffic.txt.
-COPY_256MIB_TRAFFIC_BYTES = int((131081.4 * 1.99982 + 262378.9) * 1024)       # 537.1 MB, 1.0004 x algorithmic
-ROPE_Q_TRAFFIC_BYTES = int((132111.6 * 1.99982 + 262145.1) * 1024)            # 539.0 MB, 1.0000 x algorithmic
-ROPE_K_TRAFFIC_BYTES = int((33807.6 * 1.99982 + 65537.0) * 1024)              # 136.3 MB, 1.0002 x algorithmic
+# Bytes per launch that cross the L2 -> fabric boundary, measured with rocprofv3 --pmc (FETCH_SIZE in
+# one run, WRITE_SIZE in another, KiB per dispatch), each scaled by what the same counter reads for
+# the runtime's own 256 MiB buffer copy in the same run (FETCH_SIZE reads 131083.5 KiB for
+# 262144 KiB fetched, so x1.99982; WRITE_SIZE reads 262144.0, so x1.0).
+# Source: profiles/sideaware_copy_256MiB_and_rope_bf16_llama3_hbm_traffic.txt.
+COPY_256MIB_TRAFFIC_BYTES = int((131081.2 * 1.99982 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
+ROPE_Q_TRAFFIC_BYTES = int((138551.0 * 1.99982 + 262144.0) * 1024)            # 552.2 MB, 1.0245 x algorithmic
+ROPE_K_TRAFFIC_BYTES = int((33807.6 * 1.99982 + 65536.0) * 1024)              # 136.3 MB, 1.0002 x algorithmic
 
 
 def log(*a):

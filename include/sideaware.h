@@ -80,7 +80,9 @@ void sideaware_compression(bool enable);              /* accepted, no effect: no
 void sideaware_alloc_threshold(size_t threshold);     /* large/small boundary of malloc_auto */
 void sideaware_prealloc_config(int extra_required, int extra_alloc); /* accepted, no effect: nothing is pre-mapped */
 void sideaware_free_mapped_thresholds(size_t start_threshold, size_t end_threshold);
-                                                      /* cached large bytes above `start` are trimmed to `end` on a miss */
+                                                      /* cached large bytes above `start` are trimmed to `end` on a miss;
+                                                         defaults: 1/5 and 1/40 of device memory (16 GiB and 2 GiB
+                                                         on parts of 80 GB or less, the reference's values) */
 void sideaware_write_sass(const char* filename);      /* append the gfx950 ISA of every later compile to this file */
 
 /* ---- queries (sideaware.cu:1492-1522) ---------------------------------------------------- */

@@ -245,6 +245,12 @@ void DeviceContext::initialize() {
 
     backing = std::make_unique<HipBacking>(device);
     pool = std::make_unique<Pool>(backing.get());
+    // The reference trims its cache from 16 GiB down to 2 GiB on an 80 GB part
+    // (sideaware.cu:421-422); keep those proportions of whatever this device holds.
+    size_t free_bytes = 0, total_bytes = 0;
+    if (hipMemGetInfo(&free_bytes, &total_bytes) == hipSuccess && total_bytes > (80ull << 30)) {
+        pool->set_trim_thresholds(total_bytes / 5, total_bytes / 40);
+    }
     apply_config(pool.get());
     ready = true;
 }
