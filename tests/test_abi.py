@@ -218,3 +218,15 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     # bf16 is narrowed by the hardware's round-to-nearest-even convert, fp32 math is not fused
     isa = _isa_of(lib, tmp_path, rope, 0)
     assert "v_cvt_pk_bf16_f32" in isa and "v_fma_f32" not in isa and "v_pk_mul_f32" not in isa
+
+
+def test_a_plain_c_program_links_and_runs_against_the_header(lib, tmp_path):
+    # the boundary is a C ABI: a C compiler (not C++) must accept include/sideaware.h and the
+    # program must link against the shared library
+    exe = tmp_path / "c_host"
+    lib_dir = os.path.dirname(sa_build.LIB_PATH)
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", os.path.join(ROOT, "tests", "native", "c_host.c"),
+                    "-L" + lib_dir, "-l:sideaware.so", "-Wl,-rpath," + lib_dir, "-o", str(exe)], check=True)
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "c host ok" in proc.stdout

@@ -275,6 +275,26 @@ def test_two_in_two_out_mixed_widths(sa, n):
     assert torch.equal(out1, (in1 * 10.0).half())
 
 
+def test_reverse_order_with_persistent_grids(sa):
+    # reverse_order walks each XCD's tiles from the end; with a fixed number of workgroups per CU the
+    # grid is persistent and every workgroup loops.  Lengths with and without a partial last tile.
+    lib = sa.library()
+    kid = sa.sideaware_create_kernel(MIXED_HEADER)          # its header sets reverse_order = true
+    stream = torch.cuda.current_stream().cuda_stream
+    for n in (4096 * 37, 4096 * 37 + 52, 1000):
+        in0 = (torch.arange(n, device="cuda", dtype=torch.float32) % 64).to(torch.bfloat16)
+        in1 = torch.full((n,), 3.0, device="cuda", dtype=torch.float32)
+        for groups, per_xcd in ((1, 1), (2, 3), (4, 0)):
+            out0 = torch.zeros(n, device="cuda", dtype=torch.float32)
+            out1 = torch.zeros(n, device="cuda", dtype=torch.float16)
+            lib.sideaware_elementwise(kid, n * 4, out0.data_ptr(), out1.data_ptr(), 0, 0, in0.data_ptr(),
+                                      in1.data_ptr(), 0, 0, 0, 0, groups, per_xcd, 0, stream)
+            torch.cuda.synchronize()
+            assert torch.equal(out0, in0.float() + in1), (n, groups, per_xcd)
+            assert torch.equal(out1, (in1 * 10.0).half()), (n, groups, per_xcd)
+    assert_no_library_error(sa)
+
+
 def test_output_only_fill(sa):
     from l2_torch_alloc_amd import ops
     out = torch.zeros(3 * MiB // 4 + 4, dtype=torch.int32, device="cuda")
