@@ -207,6 +207,31 @@ def bench_rope_fp32_gpt2(steps, warmup):
             "note": "25 MB: launch-bound and Infinity-Cache resident, not an HBM roofline case"}
 
 
+def stripe_ab(steps):
+    """A/B evidence for the stripe -> XCD map, meant to be run under `rocprofv3 --pmc FETCH_SIZE`:
+    the q RoPE with 4 KiB tiles (half a token row), once with 4 KiB ownership stripes, so the two
+    halves of a row go to two XCDs and both L2s fetch the row's table entries, and once with 16 KiB
+    and 256 KiB stripes, where a row stays on one XCD.  Kernel names carry the stripe size."""
+    import torch
+    from l2_torch_alloc_amd import headers, ops, wrapper
+    lib, stream = _abi()
+    B, T, HS = 8, 4096, 128
+    q = torch.randn(B, T, 32, HS, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    freqs = ops.freqs_cis_table(HS, T, 500000.0).cuda()
+    nbytes = q.numel() * 2
+    out = {}
+    for stripe in (4096, 16384, 262144):
+        assert lib.sideaware_tune(b"stripe_bytes", stripe) == 0
+        text = headers.rope_header(T, 32, 0, HS, "bf16", "heads", unrolled=1, stream_output=True).decode()
+        text = text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME stripe%d_" % stripe)
+        kid = wrapper.sideaware_create_kernel(text.encode())
+        sec = time_region(lambda: lib.sideaware_elementwise(kid, nbytes, q.data_ptr(), 0, 0, 0, q.data_ptr(),
+                                                            freqs.data_ptr(), 0, 0, 0, 0, 0, 0, 0, stream), steps, 2)
+        out["stripe_%d" % stripe] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes + freqs.numel() * 4, sec)}
+    assert lib.sideaware_tune(b"stripe_bytes", 16384) == 0
+    return out
+
+
 def churn_sizes(n_ops=10000, seed=4):
     rng = random.Random(seed)
     return [max(16, int(4096 * 2 ** (rng.random() * 17)) // 16 * 16) for _ in range(n_ops)]
@@ -343,6 +368,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--quick", action="store_true", help="headline copy and bf16 RoPE only")
+    ap.add_argument("--stripe-ab", action="store_true",
+                    help="only the stripe-size A/B of the q RoPE (for a FETCH_SIZE profile)")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -365,6 +392,10 @@ def main():
     wrapper.sideaware_init()
     info = wrapper.sideaware_info()
     log("device:", torch.cuda.get_device_name(0), info)
+
+    if args.stripe_ab:
+        print(json.dumps({"stripe_ab": stripe_ab(args.steps)}))
+        return
 
     copy = bench_copy(256 * MiB, args.steps, args.warmup, "uint8", seed=0)
     log("copy 256 MiB:", copy)
