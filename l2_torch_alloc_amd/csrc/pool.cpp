@@ -92,51 +92,61 @@ void* const kMixedStreams = (void*)(uintptr_t)1;
 }  // namespace
 
 // Adds a free extent, merging it with free neighbours of the same arena.
-void Pool::extent_insert_locked(uintptr_t addr, Extent e) {
+void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
+    ExtentIndex& ix = free_[kind];
     auto erase_size = [&](size_t bytes, uintptr_t a) {
-        auto range = free_by_size_.equal_range(bytes);
+        auto range = ix.by_size.equal_range(bytes);
         for (auto it = range.first; it != range.second; ++it) {
-            if (it->second == a) { free_by_size_.erase(it); return; }
+            if (it->second == a) { ix.by_size.erase(it); return; }
         }
     };
-    auto next = free_by_addr_.lower_bound(addr);
-    if (next != free_by_addr_.end() && next->second.arena == e.arena && addr + e.bytes == next->first) {
+    auto next = ix.by_addr.lower_bound(addr);
+    if (next != ix.by_addr.end() && next->second.arena == e.arena && addr + e.bytes == next->first) {
         if (next->second.stream != e.stream) e.stream = kMixedStreams;
         e.bytes += next->second.bytes;
         erase_size(next->second.bytes, next->first);
-        next = free_by_addr_.erase(next);
+        next = ix.by_addr.erase(next);
     }
-    if (next != free_by_addr_.begin()) {
+    if (next != ix.by_addr.begin()) {
         auto prev = std::prev(next);
         if (prev->second.arena == e.arena && prev->first + prev->second.bytes == addr) {
             if (prev->second.stream != e.stream) e.stream = kMixedStreams;
             addr = prev->first;
             e.bytes += prev->second.bytes;
             erase_size(prev->second.bytes, prev->first);
-            free_by_addr_.erase(prev);
+            ix.by_addr.erase(prev);
         }
     }
-    free_by_addr_[addr] = e;
-    free_by_size_.emplace(e.bytes, addr);
+    ix.by_addr[addr] = e;
+    ix.by_size.emplace(e.bytes, addr);
 }
 
-// Best fit from the free extents; the remainder stays free.  Pages that were freed on another
+// Takes `bytes` from the front of the best-fitting free extent; the remainder stays free.
+bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken) {
+    ExtentIndex& ix = free_[kind];
+    auto sit = ix.by_size.lower_bound(bytes);
+    if (sit == ix.by_size.end()) return false;
+    *addr = sit->second;
+    auto ait = ix.by_addr.find(*addr);
+    *taken = ait->second;
+    ix.by_size.erase(sit);
+    ix.by_addr.erase(ait);
+    if (taken->bytes > bytes) {
+        Extent rest = *taken;
+        rest.bytes = taken->bytes - bytes;
+        ix.by_addr[*addr + bytes] = rest;
+        ix.by_size.emplace(rest.bytes, *addr + bytes);
+    }
+    (kind == kSlabArenas ? st_.bytes_free_slab_arena : st_.bytes_free_arena) -= bytes;
+    return true;
+}
+
+// Best fit from the free extents of the large regions' arenas.  Pages that were freed on another
 // stream are waited for first (stream order, as for a cached region).
 void* Pool::carve_locked(size_t rounded, void* stream) {
-    auto sit = free_by_size_.lower_bound(rounded);
-    if (sit == free_by_size_.end()) return nullptr;
-    const uintptr_t addr = sit->second;
-    auto ait = free_by_addr_.find(addr);
-    Extent e = ait->second;
-    free_by_size_.erase(sit);
-    free_by_addr_.erase(ait);
-    if (e.bytes > rounded) {
-        Extent rest = e;
-        rest.bytes = e.bytes - rounded;
-        free_by_addr_[addr + rounded] = rest;
-        free_by_size_.emplace(rest.bytes, addr + rounded);
-    }
-    st_.bytes_free_arena -= rounded;
+    uintptr_t addr;
+    Extent e;
+    if (!extent_take_locked(kLargeArenas, rounded, &addr, &e)) return nullptr;
     if (e.stream == kMixedStreams) {
         backing_->sync_device();
         st_.device_syncs++;
@@ -154,10 +164,12 @@ void* Pool::carve_locked(size_t rounded, void* stream) {
     return blk.ptr;
 }
 
-// A fresh arena from the backing store: the configured size, or just the request if that is
-// larger, or if the backing store cannot give the configured size any more.
-bool Pool::new_arena_locked(size_t min_bytes) {
-    size_t want = std::max(arena_bytes_, min_bytes);
+// A fresh arena from the backing store: the configured size (for slabs at most
+// kMaxSlabArenaBytes), or just the request if that is larger, or if the backing store cannot
+// give the configured size any more.
+bool Pool::new_arena_locked(int kind, size_t min_bytes) {
+    size_t configured = kind == kSlabArenas ? std::min(arena_bytes_, kMaxSlabArenaBytes) : arena_bytes_;
+    size_t want = std::max(configured, min_bytes);
     void* p = backing_acquire_locked(want);
     if (!p && want > min_bytes) {
         want = min_bytes;
@@ -170,12 +182,13 @@ bool Pool::new_arena_locked(size_t min_bytes) {
     auto arena = std::make_unique<Arena>();
     arena->base = (char*)p;
     arena->bytes = want;
+    arena->for_slabs = kind == kSlabArenas;
     Extent e;
     e.bytes = want;
     e.arena = arena.get();
     e.stream = nullptr;            // never used: nothing to wait for
-    st_.bytes_free_arena += want;
-    extent_insert_locked((uintptr_t)p, e);
+    (kind == kSlabArenas ? st_.bytes_free_slab_arena : st_.bytes_free_arena) += want;
+    extent_insert_locked(kind, (uintptr_t)p, e);
     arenas_.push_back(std::move(arena));
     return true;
 }
@@ -189,36 +202,39 @@ void Pool::flush_cache_locked() {
             e.arena = blk.arena;
             e.stream = blk.last_stream;
             st_.bytes_free_arena += blk.bytes;
-            extent_insert_locked((uintptr_t)blk.ptr, e);
+            extent_insert_locked(kLargeArenas, (uintptr_t)blk.ptr, e);
         }
     }
     large_cache_.clear();
     st_.bytes_cached_large = 0;
 }
 
-// Returns wholly free arenas to the backing store until at most `down_to` free bytes remain in
-// arenas.  The device is drained first (unmap_free_allocations does the same,
-// sideaware.cu:873-906): freed pages may still be in use by work queued before the free.
-size_t Pool::release_free_arenas_locked(size_t down_to) {
+// Returns wholly free arenas of one kind to the backing store until at most `down_to` free bytes
+// remain in that kind's arenas.  The device is drained first (unmap_free_allocations does the
+// same, sideaware.cu:873-906): freed pages may still be in use by work queued before the free.
+size_t Pool::release_free_arenas_locked(int kind, size_t down_to, bool device_idle) {
+    ExtentIndex& ix = free_[kind];
+    uint64_t& free_bytes = kind == kSlabArenas ? st_.bytes_free_slab_arena : st_.bytes_free_arena;
     size_t released = 0;
-    bool synced = false;
-    for (auto it = arenas_.begin(); it != arenas_.end() && st_.bytes_free_arena > down_to;) {
+    bool synced = device_idle;
+    for (auto it = arenas_.begin(); it != arenas_.end() && free_bytes > down_to;) {
         Arena* a = it->get();
-        auto fit = free_by_addr_.find((uintptr_t)a->base);
-        if (fit == free_by_addr_.end() || fit->second.bytes != a->bytes) { ++it; continue; }
+        if (a->for_slabs != (kind == kSlabArenas)) { ++it; continue; }
+        auto fit = ix.by_addr.find((uintptr_t)a->base);
+        if (fit == ix.by_addr.end() || fit->second.bytes != a->bytes) { ++it; continue; }
         if (!synced) {
             backing_->sync_device();
             st_.device_syncs++;
             synced = true;
         }
-        auto range = free_by_size_.equal_range(a->bytes);
+        auto range = ix.by_size.equal_range(a->bytes);
         for (auto sit = range.first; sit != range.second; ++sit) {
-            if (sit->second == (uintptr_t)a->base) { free_by_size_.erase(sit); break; }
+            if (sit->second == (uintptr_t)a->base) { ix.by_size.erase(sit); break; }
         }
-        free_by_addr_.erase(fit);
+        ix.by_addr.erase(fit);
         backing_->release(a->base, a->bytes);
         st_.backing_releases++;
-        st_.bytes_free_arena -= a->bytes;
+        free_bytes -= a->bytes;
         note_reserved(-(int64_t)a->bytes);
         released += a->bytes;
         it = arenas_.erase(it);
@@ -230,7 +246,7 @@ size_t Pool::release_free_arenas_locked(size_t down_to) {
 size_t Pool::trim_large_locked(size_t down_to) {
     if (st_.bytes_cached_large + st_.bytes_free_arena <= down_to) return 0;
     flush_cache_locked();
-    return release_free_arenas_locked(down_to);
+    return release_free_arenas_locked(kLargeArenas, down_to);
 }
 
 void* Pool::allocate_large_locked(size_t bytes, void* stream) {
@@ -274,20 +290,20 @@ void* Pool::allocate_large_locked(size_t bytes, void* stream) {
         st_.trims++;
         if (void* p = carve_locked(rounded, stream)) return p;
     }
-    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
+    if (new_arena_locked(kLargeArenas, rounded)) return carve_locked(rounded, stream);
 
     // 5) the backing store refused: fold the cache back, carve if that made room, else give every
     //    free arena back and retry
     st_.ladder_retries++;
     flush_cache_locked();
     if (void* p = carve_locked(rounded, stream)) return p;
-    release_free_arenas_locked(0);
-    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
+    release_free_arenas_locked(kLargeArenas, 0);
+    if (new_arena_locked(kLargeArenas, rounded)) return carve_locked(rounded, stream);
 
     // 6) give back empty slabs too and retry one last time
     st_.ladder_retries++;
     release_empty_slabs_locked();
-    if (new_arena_locked(rounded)) return carve_locked(rounded, stream);
+    if (new_arena_locked(kLargeArenas, rounded)) return carve_locked(rounded, stream);
 
     st_.failures++;
     return nullptr;
@@ -297,25 +313,50 @@ void* Pool::allocate_large_locked(size_t bytes, void* stream) {
 // Small path
 // ---------------------------------------------------------------------------------------------
 
+// Memory for one slab: carved from the slabs' arenas (a new one when none has room), or a
+// backing allocation of its own when arenas are switched off.  Extents in the slabs' arenas are
+// only ever freed after a device sync, so a carve there never has a stream to wait for.
+void* Pool::slab_memory_locked(size_t bytes, Arena** arena) {
+    *arena = nullptr;
+    if (arena_bytes_ == 0) {
+        void* p = backing_acquire_locked(bytes);
+        if (p) note_reserved((int64_t)bytes);
+        return p;
+    }
+    uintptr_t addr;
+    Extent e;
+    if (!extent_take_locked(kSlabArenas, bytes, &addr, &e)) {
+        if (!new_arena_locked(kSlabArenas, bytes)) return nullptr;
+        if (!extent_take_locked(kSlabArenas, bytes, &addr, &e)) return nullptr;
+    }
+    *arena = e.arena;
+    return (void*)addr;
+}
+
 Pool::Slab* Pool::new_slab_locked(size_t block) {
     size_t want = std::min(std::max(block * 16, kRegionAlign), kMaxSlabBytes);
     want = std::max(want, block);
     size_t bytes = round_large(want);
-    void* p = backing_acquire_locked(bytes);
+    Arena* arena = nullptr;
+    void* p = slab_memory_locked(bytes, &arena);
     if (!p) {
         // the same ladder as the large path, compressed: drop caches, then retry once
         st_.ladder_retries++;
         trim_large_locked(0);
         release_empty_slabs_locked();
-        p = backing_acquire_locked(bytes);
+        p = slab_memory_locked(bytes, &arena);
+        if (!p && round_large(block) < bytes) {
+            bytes = round_large(block);      // last resort: a slab of a single block
+            p = slab_memory_locked(bytes, &arena);
+        }
         if (!p) return nullptr;
     }
-    note_reserved((int64_t)bytes);
     st_.slabs_acquired++;
     auto slab = std::make_unique<Slab>();
     slab->base = (char*)p;
     slab->bytes = bytes;
     slab->block = block;
+    slab->arena = arena;
     slab->capacity = (uint32_t)(bytes / block);
     slab->in_use.assign(slab->capacity, 0);
     for (size_t off = 0; off < bytes; off += kRegionAlign) {
@@ -364,8 +405,9 @@ void* Pool::allocate_small_locked(size_t bytes, void* stream) {
     return p;
 }
 
-// Gives back every slab with no live block.  Their blocks are purged from the class free lists
-// first; a slab that is only partly used stays.
+// Gives back every slab with no live block, and then every arena of slabs that is wholly free;
+// returns the bytes that went back to the backing store.  The slabs' blocks are purged from the
+// class free lists first; a slab that is only partly used stays.
 size_t Pool::release_empty_slabs_locked() {
     bool any = false;
     for (auto& s : slab_store_) any |= (s->live == 0);
@@ -397,13 +439,23 @@ size_t Pool::release_empty_slabs_locked() {
         for (size_t off = 0; off < s->bytes; off += kRegionAlign) {
             slab_by_page_.erase(((uintptr_t)s->base + off) / kRegionAlign);
         }
-        backing_->release(s->base, s->bytes);
-        st_.backing_releases++;
         st_.bytes_cached_small -= (uint64_t)s->capacity * s->block;
-        note_reserved(-(int64_t)s->bytes);
-        released += s->bytes;
+        if (s->arena) {
+            Extent e;
+            e.bytes = s->bytes;
+            e.arena = s->arena;
+            e.stream = nullptr;        // the device was drained above
+            st_.bytes_free_slab_arena += s->bytes;
+            extent_insert_locked(kSlabArenas, (uintptr_t)s->base, e);
+        } else {
+            backing_->release(s->base, s->bytes);
+            st_.backing_releases++;
+            note_reserved(-(int64_t)s->bytes);
+            released += s->bytes;
+        }
         it = slab_store_.erase(it);
     }
+    released += release_free_arenas_locked(kSlabArenas, 0, /*device_idle=*/true);
     return released;
 }
 

@@ -20,7 +20,9 @@
 //          (sideaware.cu:1233-1252);
 //   small  (size <  threshold): 512 B-granular size classes carved from slabs, so the common
 //          small request never reaches the driver (the reference forwards these to
-//          cudaMallocAsync, sideaware.cu:1326-1339).
+//          cudaMallocAsync, sideaware.cu:1326-1339).  Slabs are themselves carved from arenas
+//          of their own (up to 1 GiB each), kept apart from the large regions' arenas so that a
+//          long-lived small block never pins a multi-GiB arena.
 //
 // All device interaction goes through the Backing interface, so every policy decision in here
 // runs on a CPU with a fake backing (tests/test_pool.py).  One mutex guards all state: the
@@ -41,6 +43,7 @@ constexpr size_t kRegionAlign = 2ull << 20;      // alignment and rounding of la
 constexpr size_t kSmallGranule = 512;            // alignment and minimum size of small blocks
 constexpr size_t kMaxSlabBytes = 64ull << 20;
 constexpr size_t kDefaultArenaBytes = 4ull << 30;
+constexpr size_t kMaxSlabArenaBytes = 1ull << 30;
 
 // Where the bytes come from.  The HIP implementation lives in hip_backing.cpp.
 class Backing {
@@ -77,8 +80,9 @@ struct PoolStats {
     uint64_t bytes_reserved = 0;    // everything held from the backing store
     uint64_t peak_reserved = 0;
     uint64_t large_carves = 0;      // large requests carved from an arena's free extents
-    uint64_t arenas_acquired = 0;
-    uint64_t bytes_free_arena = 0;  // free extents inside arenas
+    uint64_t arenas_acquired = 0;   // arenas for large regions and arenas for slabs
+    uint64_t bytes_free_arena = 0;  // free extents inside the large regions' arenas
+    uint64_t bytes_free_slab_arena = 0;  // free extents inside the slabs' arenas
 };
 constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
 
@@ -121,6 +125,7 @@ private:
     struct Arena {
         char* base = nullptr;
         size_t bytes = 0;
+        bool for_slabs = false;
     };
     struct LargeBlock {
         void* ptr = nullptr;
@@ -140,8 +145,14 @@ private:
         uint32_t capacity = 0;     // blocks in the slab
         uint32_t carved = 0;       // blocks ever handed out from the bump pointer
         uint32_t live = 0;
+        Arena* arena = nullptr;    // null: a backing allocation of its own
         std::vector<uint8_t> in_use;   // one flag per block: catches double frees
     };
+    struct ExtentIndex {           // the free extents of one kind of arena, by address and by size
+        std::map<uintptr_t, Extent> by_addr;
+        std::multimap<size_t, uintptr_t> by_size;
+    };
+    enum { kLargeArenas = 0, kSlabArenas = 1 };
     struct FreeSmall {
         void* ptr;
         void* stream;
@@ -155,10 +166,12 @@ private:
     void* allocate_large_locked(size_t bytes, void* stream);
     void* allocate_small_locked(size_t bytes, void* stream);
     void* carve_locked(size_t rounded, void* stream);
-    void extent_insert_locked(uintptr_t addr, Extent e);
-    bool new_arena_locked(size_t min_bytes);
+    void extent_insert_locked(int kind, uintptr_t addr, Extent e);
+    bool extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken);
+    bool new_arena_locked(int kind, size_t min_bytes);
     void flush_cache_locked();
-    size_t release_free_arenas_locked(size_t down_to);
+    size_t release_free_arenas_locked(int kind, size_t down_to, bool device_idle = false);
+    void* slab_memory_locked(size_t bytes, Arena** arena);
     Slab* new_slab_locked(size_t block);
     size_t trim_large_locked(size_t down_to);
     size_t release_empty_slabs_locked();
@@ -176,8 +189,7 @@ private:
     std::map<size_t, std::vector<LargeBlock>> large_cache_;            // rounded size -> LIFO, sizes ordered
     std::unordered_map<void*, LargeBlock> large_live_;
     std::vector<std::unique_ptr<Arena>> arenas_;
-    std::map<uintptr_t, Extent> free_by_addr_;
-    std::multimap<size_t, uintptr_t> free_by_size_;
+    ExtentIndex free_[2];                                              // kLargeArenas, kSlabArenas
     std::vector<SmallClass> small_;                                    // class index -> state
     std::unordered_map<uintptr_t, Slab*> slab_by_page_;                // addr >> 21 -> slab
     std::vector<std::unique_ptr<Slab>> slab_store_;

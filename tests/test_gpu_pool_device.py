@@ -73,7 +73,8 @@ def test_release_unused_gives_memory_back(sa):
     # an arena that still holds a live region stays
     assert after["bytes_cached_large"] == 0
     assert after["bytes_reserved"] == before["bytes_reserved"] - freed
-    assert after["bytes_free_arena"] + after["bytes_live"] + after["bytes_cached_small"] <= after["bytes_reserved"]
+    assert (after["bytes_free_arena"] + after["bytes_free_slab_arena"] + after["bytes_live"]
+            + after["bytes_cached_small"]) <= after["bytes_reserved"]
 
 
 def test_out_of_memory_is_a_null_pointer_not_a_crash(sa):

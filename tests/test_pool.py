@@ -26,7 +26,7 @@ GiB = 1 << 30
 FIELDS = ("large_hits", "large_misses", "small_hits", "small_carves", "slabs_acquired", "backing_acquires",
           "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
           "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
-          "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena")
+          "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena")
 
 
 def build_harness():
@@ -357,6 +357,67 @@ def test_carved_pages_wait_for_the_stream_that_freed_them(ph):
         pool.close()
 
 
+def test_slabs_are_carved_from_their_own_arenas(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        big = pool.alloc(16 * MiB)
+        smalls = [pool.alloc(n) for n in (1000, 5000, 70000, 300000, 3 * MiB)]   # five classes, five slabs
+        assert all(smalls)
+        st = pool.stats()
+        assert st["slabs_acquired"] == 5
+        # one arena for the large region, one for all five slabs: two driver calls, not six
+        assert pool.log() == ["acquire %d" % (64 * MiB), "acquire %d" % (64 * MiB)]
+        assert st["arenas_acquired"] == 2 and st["backing_acquires"] == 2
+        # slabs never share an arena with large regions: all five sit in one 64 MiB window, `big` outside it
+        lo = min(smalls)
+        assert all(lo <= s < lo + 64 * MiB for s in smalls) and not (lo <= big < lo + 64 * MiB)
+        # 2 + 2 + 2 + 6 + 48 MiB of slabs (16 blocks each, at least 2 MiB, at most 64 MiB): 60 MiB carved
+        assert st["bytes_free_slab_arena"] == 64 * MiB - 60 * MiB
+        # emptied slabs go back to their arena; the arena goes home once all of it is free
+        for s in smalls[:-1]:
+            pool.free(s)
+        assert pool.L.ph_release_unused(pool.h) == 0               # the 3 MiB block still pins the arena
+        assert pool.stats()["bytes_free_slab_arena"] == 64 * MiB - 48 * MiB
+        again = pool.alloc(1000)                                   # carved from the arena again: no driver call
+        assert again and pool.stats()["backing_acquires"] == 2
+        pool.free(again)
+        pool.free(smalls[-1])
+        assert pool.L.ph_release_unused(pool.h) == 64 * MiB
+        assert pool.stats()["bytes_free_slab_arena"] == 0
+        assert pool.L.ph_backing_live_blocks(pool.h) == 1          # only the large region's arena
+        assert pool.L.ph_owns(pool.h, big)
+    finally:
+        pool.close()
+
+
+def test_slab_arena_size_is_capped(ph):
+    pool = P(ph, capacity=16 * GiB, arena=4 * GiB)
+    try:
+        assert pool.alloc(4096)
+        assert pool.log() == ["acquire %d" % (1 * GiB)]            # not the 4 GiB of a large-region arena
+    finally:
+        pool.close()
+
+
+def test_slab_falls_back_when_the_backing_is_short(ph):
+    pool = P(ph, capacity=40 * MiB, arena=64 * MiB)
+    try:
+        a = pool.alloc(4096)                                        # no 64 MiB arena fits: a 2 MiB one
+        assert a and pool.log() == ["acquire_failed %d" % (64 * MiB), "acquire %d" % (2 * MiB)]
+        big = pool.alloc(30 * MiB)
+        assert big
+        pool.free(big)
+        pool.clear_log()
+        b = pool.alloc(5 * MiB)         # its class wants a 64 MiB slab, more than the device has left
+        # the cache is given back first; when 64 MiB still does not fit, a slab of one block does
+        assert b and pool.stats()["failures"] == 0
+        log = pool.log()
+        assert "release %d" % (30 * MiB) in log and log[-1] == "acquire %d" % (6 * MiB)
+        assert pool.L.ph_block_bytes(pool.h, b) == 5 * MiB
+    finally:
+        pool.close()
+
+
 # ------------------------------------------------------------------------------ small path
 
 def test_small_blocks_are_pooled_and_512_aligned(pool):
@@ -429,7 +490,7 @@ def test_random_churn_keeps_blocks_disjoint_and_accounts_balance(ph, arena):
                 assert st["bytes_live"] == sum(live.values())
                 assert st["bytes_reserved"] == pool.L.ph_backing_used(pool.h)
                 assert (st["bytes_live"] + st["bytes_cached_large"] + st["bytes_cached_small"]
-                        + st["bytes_free_arena"]) <= st["bytes_reserved"]
+                        + st["bytes_free_arena"] + st["bytes_free_slab_arena"]) <= st["bytes_reserved"]
         for p in list(live):
             assert pool.free(p) == 0
         st = pool.stats()
