@@ -392,7 +392,21 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
     }
     ScopedDevice guard(ctx->device);
     hipError_t err = hipModuleLoadData(&k.module, r.code.data());
-    if (err == hipSuccess) err = hipModuleGetFunction(&k.fn, k.module, e.function_name.c_str());
+    if (err == hipSuccess) {
+        // The module itself says what its entry point is called: the header text may not (a
+        // header that is only `#include "file"`, example_llmc_rope.cu:138).
+        char name[128] = {0};
+        hipDeviceptr_t name_ptr = nullptr;
+        size_t name_bytes = 0;
+        if (hipModuleGetGlobal(&name_ptr, &name_bytes, k.module, "sideaware_kernel_name") == hipSuccess &&
+            name_bytes > 1 && name_bytes < sizeof name &&
+            hipMemcpyDtoH(name, name_ptr, name_bytes) == hipSuccess && name[0]) {
+            e.function_name = name;               // the registry lock is held
+        } else {
+            (void)hipGetLastError();
+        }
+        err = hipModuleGetFunction(&k.fn, k.module, e.function_name.c_str());
+    }
     if (err != hipSuccess) {
         k.failed = true;
         k.fn = nullptr;

@@ -169,6 +169,22 @@ def test_broken_header_reports_instead_of_aborting(lib):
     assert rc != 0 and "error" in log
 
 
+def test_header_may_include_a_file_relative_to_the_working_directory(lib, tmp_path, monkeypatch):
+    # example_llmc_rope.cu:138 registers the one-line header `#include "kernel_rope.cuh"` and relies
+    # on the compiler finding the file in the process's working directory
+    (tmp_path / "my_rope_op.h").write_bytes(headers.rope_header(1024, 32, 32, 128, "fp32", "qkv"))
+    monkeypatch.chdir(tmp_path)
+    rc, log = compile_ok(lib, b'#include "my_rope_op.h"\n', 0)
+    assert rc == 0, log
+    # the file's content is read at every compile, never served from the on-disk cache: a changed
+    # file must not keep compiling as the old one
+    (tmp_path / "my_rope_op.h").write_bytes(b"typedef int o0; this is not C++")
+    rc, log = compile_ok(lib, b'#include "my_rope_op.h"\n', 0)
+    assert rc != 0 and "error" in log
+    rc, log = compile_ok(lib, b'#include "no_such_file.h"\n', 0)
+    assert rc != 0 and "no_such_file.h" in log
+
+
 REFERENCE_DIR = "/root/reference"
 
 
