@@ -71,9 +71,23 @@ void HipBacking::sync_device() {
     (void)hipDeviceSynchronize();
 }
 
-void HipBacking::sync_stream(void* stream) {
+// The consumer stream waits, on the device, for what the producer stream has queued so far; the
+// host does not block.  If the event cannot be made or recorded the host waits for the producer
+// stream instead, and if even that is refused, for the whole device.
+void HipBacking::order_after(void* producer, void* consumer) {
     DeviceGuard g(device_);
-    (void)hipStreamSynchronize((hipStream_t)stream);
+    hipEvent_t ev = nullptr;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess) {
+        bool ordered = hipEventRecord(ev, (hipStream_t)producer) == hipSuccess &&
+                       hipStreamWaitEvent((hipStream_t)consumer, ev, 0) == hipSuccess;
+        (void)hipEventDestroy(ev);      // released by the runtime once the wait has been satisfied
+        if (ordered) return;
+    }
+    (void)hipGetLastError();
+    if (hipStreamSynchronize((hipStream_t)producer) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipDeviceSynchronize();
+    }
 }
 
 int HipBacking::free_foreign(void* ptr, void* stream) {

@@ -14,7 +14,7 @@ public:
     void* acquire(size_t bytes) override;
     void release(void* ptr, size_t bytes) override;
     void sync_device() override;
-    void sync_stream(void* stream) override;
+    void order_after(void* producer, void* consumer) override;
     int free_foreign(void* ptr, void* stream) override;
 
 private:

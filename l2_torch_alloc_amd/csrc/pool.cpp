@@ -151,7 +151,7 @@ void* Pool::carve_locked(size_t rounded, void* stream) {
         backing_->sync_device();
         st_.device_syncs++;
     } else if (e.stream != stream && e.stream != nullptr) {
-        backing_->sync_stream(e.stream);
+        backing_->order_after(e.stream, stream);
         st_.stream_syncs++;
     }
     LargeBlock blk;
@@ -271,7 +271,7 @@ void* Pool::allocate_large_locked(size_t bytes, void* stream) {
         if (it->second.empty()) large_cache_.erase(it);
         st_.bytes_cached_large -= blk.bytes;
         if (blk.last_stream != stream) {
-            backing_->sync_stream(blk.last_stream);
+            backing_->order_after(blk.last_stream, stream);
             st_.stream_syncs++;
             blk.last_stream = stream;
         }
@@ -377,7 +377,7 @@ void* Pool::allocate_small_locked(size_t bytes, void* stream) {
         FreeSmall f = cls.free.back();
         cls.free.pop_back();
         if (f.stream != stream) {
-            backing_->sync_stream(f.stream);
+            backing_->order_after(f.stream, stream);
             st_.stream_syncs++;
         }
         p = f.ptr;

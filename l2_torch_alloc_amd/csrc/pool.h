@@ -54,8 +54,11 @@ public:
     virtual void release(void* ptr, size_t bytes) = 0;
     // Block until every stream of the device is idle (before memory goes back to the driver).
     virtual void sync_device() = 0;
-    // Block until `stream` is idle (before a block moves to another stream).
-    virtual void sync_stream(void* stream) = 0;
+    // A block last used on `producer` is about to be used on `consumer`: everything queued on
+    // `producer` so far must finish before anything queued on `consumer` from now on starts.
+    // (The reference blocks the host on the old stream, sideaware.cu:1209-1212; an implementation
+    // may order the two streams on the device instead.)
+    virtual void order_after(void* producer, void* consumer) = 0;
     // A pointer the pool never handed out: forward to the runtime's own free.
     virtual int free_foreign(void* ptr, void* stream) = 0;
 };
@@ -68,7 +71,7 @@ struct PoolStats {
     uint64_t slabs_acquired = 0;
     uint64_t backing_acquires = 0;
     uint64_t backing_releases = 0;
-    uint64_t stream_syncs = 0;
+    uint64_t stream_syncs = 0;      // blocks handed from one stream to another
     uint64_t device_syncs = 0;
     uint64_t trims = 0;             // threshold-driven trims of the large cache
     uint64_t ladder_retries = 0;    // times a request needed step 3 or 4 of the ladder

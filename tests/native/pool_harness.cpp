@@ -20,7 +20,7 @@ struct FakeBacking final : Backing {
     size_t used = 0;
     uintptr_t next = 0x7f0000000000ull;          // 2 MiB-aligned, far from real memory
     std::map<uintptr_t, size_t> live;
-    std::vector<std::string> log;                // "acquire N", "release N", "sync_device", "sync_stream S", "foreign P"
+    std::vector<std::string> log;                // "acquire N", "release N", "sync_device", "order A -> B", "foreign P"
     int foreign_result = 0;
 
     explicit FakeBacking(size_t cap) : capacity(cap) {}
@@ -48,7 +48,9 @@ struct FakeBacking final : Backing {
         log.push_back("release " + std::to_string(bytes));
     }
     void sync_device() override { log.push_back("sync_device"); }
-    void sync_stream(void* s) override { log.push_back("sync_stream " + std::to_string((uintptr_t)s)); }
+    void order_after(void* producer, void* consumer) override {
+        log.push_back("order " + std::to_string((uintptr_t)producer) + " -> " + std::to_string((uintptr_t)consumer));
+    }
     int free_foreign(void* p, void*) override {
         log.push_back("foreign " + std::to_string((uintptr_t)p));
         return foreign_result;

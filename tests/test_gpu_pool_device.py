@@ -188,3 +188,32 @@ def test_memcpy_under_torch_compile(sa):
     out = compiled_copy(dst, src)
     torch.cuda.synchronize()
     assert torch.equal(out, src) and torch.equal(dst, src)
+
+
+def test_block_handed_to_another_stream_waits_for_the_first(sa):
+    # Stream order (sideaware.cu:1209-1212): a block freed on stream A while A still has work
+    # queued on it, then handed to stream B, must not be touched by B before A is done with it.
+    lib = sa.library()
+    n = 256 * MiB
+    ones = torch.full((n,), 1, dtype=torch.uint8, device="cuda")
+    twos = torch.full((n,), 2, dtype=torch.uint8, device="cuda")
+    result = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    before = sa.sideaware_alloc_stats()
+    p = lib.sideaware_malloc_auto(n, 0, a.cuda_stream)
+    assert p
+    for _ in range(40):                                   # a few milliseconds of writes queued on A
+        lib.sideaware_memcpy(p, ones.data_ptr(), n, 0, a.cuda_stream)
+    lib.sideaware_free_auto(p, n, 0, a.cuda_stream)       # the host does not wait
+    q = lib.sideaware_malloc_auto(n, 0, b.cuda_stream)
+    assert q == p                                         # newest freed block of that size
+    lib.sideaware_memcpy(q, twos.data_ptr(), n, 0, b.cuda_stream)
+    torch.cuda.synchronize()
+    lib.sideaware_memcpy(result.data_ptr(), q, n, 0, None)
+    torch.cuda.synchronize()
+    assert torch.equal(result, twos)                      # B's write came last
+    after = sa.sideaware_alloc_stats()
+    assert after["stream_syncs"] == before["stream_syncs"] + 1
+    lib.sideaware_free_auto(q, n, 0, b.cuda_stream)
+    assert sa.sideaware_last_error() == ""

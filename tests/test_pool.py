@@ -174,7 +174,7 @@ def test_threshold_moves_the_boundary(pool):
     assert pool.stats()["small_carves"] == 1 and q != p
 
 
-def test_stream_handover_syncs_the_old_stream(pool):
+def test_stream_handover_orders_the_new_stream_after_the_old(pool):
     a = pool.alloc(16 * MiB, stream=11)
     pool.free(a, stream=11)
     pool.clear_log()
@@ -182,12 +182,12 @@ def test_stream_handover_syncs_the_old_stream(pool):
     assert pool.log() == []                                  # same stream: reuse is stream-ordered
     pool.free(a, stream=11)
     assert pool.alloc(16 * MiB, stream=22) == a
-    assert pool.log() == ["sync_stream 11"]
+    assert pool.log() == ["order 11 -> 22"]            # stream 22 waits for what 11 had queued
     s = pool.alloc(4096, stream=5)
     pool.free(s, stream=5)
     pool.clear_log()
     assert pool.alloc(4096, stream=6) == s
-    assert pool.log() == ["sync_stream 5"]
+    assert pool.log() == ["order 5 -> 6"]
 
 
 def test_trim_thresholds(pool):
