@@ -32,12 +32,12 @@ HBM_PEAK_GBPS = 8000.0
 
 # Bytes per launch that cross the L2 -> fabric boundary, measured with rocprofv3 --pmc (FETCH_SIZE in
 # one run, WRITE_SIZE in another, KiB per dispatch), each scaled by what the same counter reads for
-# the runtime's own 256 MiB buffer copy in the same run (FETCH_SIZE reads 131083.5 KiB for
-# 262144 KiB fetched, so x1.99982; WRITE_SIZE reads 262144.0, so x1.0).
+# the runtime's own 256 MiB buffer copy in the same run (FETCH_SIZE reads 131084.5 KiB for
+# 262144 KiB fetched, so x1.99981; WRITE_SIZE reads 262144.0, so x1.0).
 # Source: profiles/sideaware_copy_256MiB_and_rope_bf16_llama3_hbm_traffic.txt.
-COPY_256MIB_TRAFFIC_BYTES = int((131081.2 * 1.99982 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
-ROPE_Q_TRAFFIC_BYTES = int((138551.0 * 1.99982 + 262144.0) * 1024)            # 552.2 MB, 1.0245 x algorithmic
-ROPE_K_TRAFFIC_BYTES = int((33807.6 * 1.99982 + 65536.0) * 1024)              # 136.3 MB, 1.0002 x algorithmic
+COPY_256MIB_TRAFFIC_BYTES = int((131081.2 * 1.99981 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
+ROPE_Q_TRAFFIC_BYTES = int((132103.1 * 1.99981 + 262144.5) * 1024)            # 539.0 MB, 1.0000 x algorithmic
+ROPE_K_TRAFFIC_BYTES = int((33807.5 * 1.99981 + 65536.1) * 1024)              # 136.3 MB, 1.0002 x algorithmic
 
 
 def log(*a):
@@ -144,6 +144,26 @@ def bench_copy_cold(nbytes, steps):
             "after_read_scrub": {"us_median": clean * 1e6, "GBps": gbps(2 * nbytes, clean)}}
 
 
+def bench_copy_rotating(nbytes, pairs, steps):
+    """Back-to-back launches that cycle through `pairs` distinct (src, dst) pairs, so no launch
+    finds its operands in a cache (the working set is pairs * 2 * nbytes) and the only dirty
+    lines in its way are those of the launches before it: the steady state of a streaming
+    pipeline."""
+    import torch
+    srcs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+    dsts = [torch.zeros_like(t) for t in srcs]
+    lib, stream = _abi()
+    ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
+
+    def cycle():
+        for d_ptr, s_ptr in ptrs:
+            lib.sideaware_memcpy(d_ptr, s_ptr, nbytes, 0, stream)
+
+    sec = time_region(cycle, steps, 1) / pairs
+    ok = all(bool(torch.equal(d, t)) for d, t in zip(dsts, srcs))
+    return {"bytes": nbytes, "pairs": pairs, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec), "bit_exact": ok}
+
+
 def bench_rope_bf16(steps, warmup):
     """q (8,4096,32,128) and k (8,4096,8,128) bf16 in place, fp32 table theta=5e5: one step is
     the q launch followed by the k launch."""
@@ -184,7 +204,20 @@ def bench_rope_bf16(steps, warmup):
     cold_clean = statistics.median(time_each(step, 15, 1, before=lambda: words.sum()))
     del scrub, words
     total = 2 * (q_bytes + k_bytes) + table_bytes
+    # four more (q, k) sets: a cycle over five touches 1.6 GB before a tensor comes round again
+    sets = [(q, k)] + [(torch.randn_like(q), torch.randn_like(k)) for _ in range(4)]
+    set_ptrs = [(a.data_ptr(), b.data_ptr()) for a, b in sets]
+
+    def cycle():
+        for a_ptr, b_ptr in set_ptrs:
+            lib.sideaware_elementwise(kid_q, q_bytes, a_ptr, 0, 0, 0, a_ptr, fp, 0, 0, 0, 0, 0, 0, 0, stream)
+            lib.sideaware_elementwise(kid_k, k_bytes, b_ptr, 0, 0, 0, b_ptr, fp, 0, 0, 0, 0, 0, 0, 0, stream)
+
+    sec_rot = time_region(cycle, max(steps // 5, 4), 1) / len(sets)
+    del sets
     return {"bytes": total, "us": sec * 1e6, "GBps": gbps(total, sec),
+            "rotating_5_sets": {"us": sec_rot * 1e6, "GBps": gbps(total, sec_rot),
+                                "note": "steps cycle through five distinct (q, k) sets: no tensor is cache-resident"},
             "frac_of_peak": gbps(total, sec) / HBM_PEAK_GBPS,
             "roofline": {"bound": "hbm", "achieved": gbps(total, sec), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": gbps(total, sec) / HBM_PEAK_GBPS,
@@ -426,6 +459,8 @@ def main():
             log("sweep", label, sweep[label])
         also["copy_sweep_fp32"] = sweep
         also["copy_256MiB_cold_cache"] = bench_copy_cold(256 * MiB, 20)
+        also["copy_256MiB_rotating_8_pairs"] = bench_copy_rotating(256 * MiB, 8, 10)
+        log("rotating:", also["copy_256MiB_rotating_8_pairs"])
         also["alloc_raw_calls"] = bench_raw_alloc_calls()
         log("raw alloc:", also["alloc_raw_calls"])
         also["alloc_churn_sideaware"] = bench_churn(True)

@@ -295,6 +295,7 @@ static DeviceContext* get_context(int device = -1) {
 // ---------------------------------------------------------------------------------------------
 
 constexpr int kMaxDevices = 16;
+constexpr int kVariants = 8;
 
 struct CompiledKernel {
     hipModule_t module = nullptr;
@@ -311,9 +312,9 @@ struct KernelEntry {
     std::string header;
     std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`
     int default_groups = 0;     // 0: decide from occupancy
-    // [device * 4 + variant]; variant = 2*beyond_cache + wide_index.  Fixed size: launches keep
-    // pointers into it while other threads compile other variants.
-    std::array<CompiledKernel, kMaxDevices * 4> compiled;
+    // [device * kVariants + variant]; variant = wide_index | beyond_cache << 1 | in_place << 2.
+    // Fixed size: launches keep pointers into it while other threads compile other variants.
+    std::array<CompiledKernel, kMaxDevices * kVariants> compiled;
 };
 
 static std::mutex g_kernels_mu;
@@ -350,6 +351,7 @@ static std::string config_block(int variant, int num_xcds, int num_cus) {
     s += "#define MAX_SM " + std::to_string(num_cus) + "\n";
     s += "#define HASH " + std::to_string((stripe_hash_mask(num_xcds) | (1 << 21)) / 16) + "\n";
     s += "#define SA_BEYOND_CACHE " + std::to_string((variant >> 1) & 1) + "\n";
+    s += "#define SA_IN_PLACE " + std::to_string((variant >> 2) & 1) + "\n";
     s += (variant & 1) ? "using size_type = long long;\nconstexpr bool aligned_2MiB = false;\n"
                        : "using size_type = int;\nconstexpr bool aligned_2MiB = true;\n";
     return s;
@@ -373,7 +375,7 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
         set_error("device %d is beyond the %d devices this build keeps kernels for", ctx->device, kMaxDevices);
         return nullptr;
     }
-    CompiledKernel& k = e.compiled[(size_t)ctx->device * 4 + (size_t)(variant & 3)];
+    CompiledKernel& k = e.compiled[(size_t)ctx->device * kVariants + (size_t)(variant & (kVariants - 1))];
     unsigned gen = g_tune_generation.load();
     if (k.generation != gen) {
         if (k.module) (void)hipModuleUnload(k.module);
@@ -532,7 +534,7 @@ int sideaware_create_kernel_advanced(const char* header, bool precompile, int de
     int id = register_header(header, default_num_groups);
     if (precompile) {
         if (DeviceContext* ctx = get_context()) {
-            for (int v = 0; v < 4; v++) get_kernel(ctx, id, v);
+            for (int v = 0; v < 4; v++) get_kernel(ctx, id, v);      // the in-place class compiles on first use
         }
     }
     return id;
@@ -557,13 +559,17 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         return;
     }
 
-    // Four instantiations per op.  Index width: 32-bit below 2 GiB, 64-bit from there on (the
+    // Lazily compiled instantiations per op.  Index width: 32-bit below 2 GiB, 64-bit from there on (the
     // reference also sends bases that are not 2 MiB-aligned to its 64-bit variant,
     // sideaware.cu:1386-1388; here the base only shifts the planner's b0, whatever its alignment).
     // Cache class: arrays whose result fits the Infinity Cache (written plainly, so the next kernel
     // finds it there) and larger ones (everything streams).
+    // In place (o0 written over i0) is a class of its own below the cache size: see the template's
+    // notes on cache policy.  Beyond it everything streams already.
     const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
-    const int variant = wide | (num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0);
+    const int beyond = num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0;
+    const int in_place = (!beyond && out0 != nullptr && out0 == in0) ? 4 : 0;
+    const int variant = wide | beyond | in_place;
 
     CompiledKernel* k = get_kernel(ctx, kernel_id, variant);
     if (!k) return;
@@ -746,7 +752,7 @@ void sideaware_clear_error(void) {
 
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity) {
     std::string hdr = header && *header ? header : kMemcpyHeader;
-    CompileResult r = compile_for_gfx950(full_source(hdr, variant & 3, kDefaultXcds, kDefaultCUs));
+    CompileResult r = compile_for_gfx950(full_source(hdr, variant & (kVariants - 1), kDefaultXcds, kDefaultCUs));
     if (log && log_capacity) {
         std::snprintf(log, log_capacity, "%s", r.log.c_str());
     }
@@ -758,16 +764,17 @@ const char* sideaware_memcpy_header(void) { return kMemcpyHeader; }
 
 const char* sideaware_config_block(int variant) {
     static std::mutex mu;
-    static std::string text[4];
+    static std::string text[kVariants];
     std::lock_guard<std::mutex> g(mu);
-    text[variant & 3] = config_block(variant & 3, kDefaultXcds, kDefaultCUs);
-    return text[variant & 3].c_str();
+    const int v = variant & (kVariants - 1);
+    text[v] = config_block(v, kDefaultXcds, kDefaultCUs);
+    return text[v].c_str();
 }
 
 int sideaware_kernel_info(int kernel_id, int variant, int* out) {
     DeviceContext* ctx = get_context();
     if (!ctx || !out) return 1;
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & 3);
+    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & (kVariants - 1));
     if (!k) return 1;
     int groups;
     {

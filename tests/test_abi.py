@@ -129,7 +129,7 @@ SHIPPED_HEADERS = {
 
 
 @pytest.mark.parametrize("name", sorted(SHIPPED_HEADERS))
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 def test_shipped_headers_compile_for_gfx950(lib, name, variant):
     rc, log = compile_ok(lib, SHIPPED_HEADERS[name], variant)
     assert rc == 0, log
@@ -219,10 +219,15 @@ def _memory_ops(isa, kernel):
 
 def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     # the built-in copy: 16-byte loads and stores; the source is marked evict
+    assert b"#define SA_IN_PLACE 0" in lib.sideaware_config_block(0)
+    assert b"#define SA_IN_PLACE 1" in lib.sideaware_config_block(4)
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 0), "sideaware_copy")
     assert loads and stores
     assert all(" nt" in l for l in loads), loads            # read once: nontemporal
     assert not any(" nt" in s for s in stores), stores        # fits the Infinity Cache: kept for the consumer
+    # in place (variant bit 2) with an evict-marked input: the stores stream as well
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 4), "sideaware_copy")
+    assert all(" nt" in l for l in loads) and all(" nt" in s for s in stores)
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 2), "sideaware_copy")
     assert all(" nt" in l for l in loads) and all(" nt" in s for s in stores)   # larger: everything streams
     # RoPE: the activations stream, the gathered table never does
@@ -231,6 +236,11 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
                                 "sideaware_rope_fwd_bf16_heads_t4096_h32_0_d128")
     assert sum(" nt" in l for l in loads) == 2 and sum(" nt" not in l for l in loads) == 4, loads
     assert all(" nt" in s for s in stores)
+    # a header that fixes the store policy itself gets exactly that, in place or not
+    fixed = headers.rope_header(4096, 32, 0, 128, "bf16", "heads", unrolled=1, stream_output=False)
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, fixed, 4),
+                                "sideaware_rope_fwd_bf16_heads_t4096_h32_0_d128")
+    assert stores and not any(" nt" in s for s in stores)
     # bf16 is narrowed by the hardware's round-to-nearest-even convert, fp32 math is not fused
     isa = _isa_of(lib, tmp_path, rope, 0)
     assert "v_cvt_pk_bf16_f32" in isa and "v_fma_f32" not in isa and "v_pk_mul_f32" not in isa
