@@ -483,3 +483,67 @@ def test_rope_bf16_packed_gqa_vs_oracle(sa):
     want = xb.copy()
     want[:, :, :Nq + Nkv] = O.rope_forward_heads_bf16(np.ascontiguousarray(xb[:, :, :Nq + Nkv]), freqs_h)
     assert np.array_equal(bits(x), want)
+
+
+def _oracle_rope(x_f32, freqs, layout, n_q, n_kv, backward):
+    if layout == "qkv":
+        fn = O.rope_backward_qkv_f32 if backward else O.rope_forward_qkv_f32
+        return fn(x_f32, freqs, n_q, n_kv)
+    fn = O.rope_backward_heads_f32 if backward else O.rope_forward_heads_f32
+    return fn(x_f32, freqs)
+
+
+def _random_rope_cases(count, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    while len(cases) < count:
+        dtype = rng.choice(["fp32", "bf16"])
+        layout = rng.choice(["qkv", "heads"])
+        head_dim = rng.choice([8, 16, 32, 64, 128, 256] if dtype == "bf16" else [4, 8, 12, 64, 96, 128])
+        n_q = rng.randint(1, 8)
+        n_kv = rng.randint(1, n_q) if layout == "qkv" else 0
+        cases.append(dict(dtype=dtype, layout=layout, head_dim=head_dim, n_q=n_q, n_kv=n_kv,
+                          B=rng.randint(1, 3), T=rng.choice([1, 2, 7, 33, 64, 100, 257]),
+                          backward=rng.random() < 0.4, in_place=rng.random() < 0.5,
+                          theta=rng.choice([10000.0, 500000.0]), scaled=rng.random() < 0.3,
+                          seed=1000 + len(cases)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_rope_cases(16, seed=20), ids=lambda c: "%s-%s-d%d-q%d-kv%d-B%d-T%d%s%s" % (
+    c["dtype"], c["layout"], c["head_dim"], c["n_q"], c["n_kv"], c["B"], c["T"],
+    "-bwd" if c["backward"] else "", "-inplace" if c["in_place"] else ""))
+def test_rope_random_shapes_vs_oracle(sa, case):
+    # Seeded random shapes, ragged against every tile size: head counts that are not powers of two,
+    # T = 1, head_dim down to one vector per head, grouped k/v heads, forward and backward, in place
+    # and out of place, both dtypes.  Bit for bit against the oracle (bf16: the oracle's fp32
+    # arithmetic on the widened inputs, narrowed round-to-nearest-even).
+    from l2_torch_alloc_amd import ops
+    c = case
+    heads = c["n_q"] + 2 * c["n_kv"] if c["layout"] == "qkv" else c["n_q"]
+    gen = torch.Generator().manual_seed(c["seed"])
+    xh = torch.randn(c["B"], c["T"], heads, c["head_dim"], generator=gen)
+    if c["dtype"] == "bf16":
+        xh = xh.to(torch.bfloat16)
+    freqs_h = O.freqs_cis(c["head_dim"], c["T"], c["theta"], c["scaled"])
+    want = _oracle_rope(xh.float().numpy(), freqs_h, c["layout"], c["n_q"], c["n_kv"], c["backward"])
+    x = xh.cuda()
+    freqs = torch.from_numpy(freqs_h).cuda()
+    out = None if c["in_place"] else torch.full_like(x, 7.0)
+    fn = {("qkv", False): ops.rope_forward_qkv, ("qkv", True): ops.rope_backward_qkv,
+          ("heads", False): ops.rope_forward_heads, ("heads", True): ops.rope_backward_heads}[(c["layout"], c["backward"])]
+    got = fn(x, freqs, c["n_q"], c["n_kv"], out=out) if c["layout"] == "qkv" else fn(x, freqs, out=out)
+    torch.cuda.synchronize()
+    rotated = c["n_q"] + c["n_kv"] if c["layout"] == "qkv" else heads
+    got_h = got.cpu()
+    if c["dtype"] == "bf16":
+        assert np.array_equal(bits(got_h[:, :, :rotated]), O.f32_to_bf16(want[:, :, :rotated]))
+    else:
+        assert np.array_equal(bits(got_h[:, :, :rotated]), want[:, :, :rotated].view(np.uint32))
+    if rotated < heads:
+        # value heads: untouched in place, carried over bit for bit out of place (as the oracle does)
+        assert np.array_equal(bits(got_h[:, :, rotated:]), bits(xh[:, :, rotated:]))
+    if not c["in_place"]:
+        assert torch.equal(x.cpu(), xh)                     # the input is left alone
+    assert_no_library_error(sa)
