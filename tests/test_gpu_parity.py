@@ -547,3 +547,43 @@ def test_rope_random_shapes_vs_oracle(sa, case):
     if not c["in_place"]:
         assert torch.equal(x.cpu(), xh)                     # the input is left alone
     assert_no_library_error(sa)
+
+
+def test_host_threads_compile_and_launch_concurrently(sa):
+    # The reference has no locking at all; here the registry and the compile cache are guarded.
+    # Six host threads each register an op of their own (new text: a fresh compile), launch it on a
+    # stream of their own next to a copy, and check the result.
+    import threading
+    from l2_torch_alloc_amd import headers
+    lib = sa.library()
+    n = 3 * MiB + 48
+    errors = []
+
+    def worker(tid):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                src = torch.full((n // 4,), tid + 1, dtype=torch.int32, device="cuda")
+                dst = torch.zeros_like(src)
+                filled = torch.zeros_like(src)
+            text = headers.fill_header().replace(b"sideaware_fill_int32", b"sideaware_fill_thread%d" % tid)
+            text = text.replace(b"out0 = sideband;", b"out0 = sideband + %d;" % (100 * tid))
+            kid = lib.sideaware_create_kernel(text)
+            assert kid > 0
+            for _ in range(20):
+                lib.sideaware_memcpy(dst.data_ptr(), src.data_ptr(), n, 0, stream.cuda_stream)
+                lib.sideaware_elementwise(kid, n, filled.data_ptr(), 0, 0, 0, 0, 0, 0, 0, 0, 5, 0, 0, 0,
+                                          stream.cuda_stream)
+            stream.synchronize()
+            assert torch.equal(dst, src), "copy on thread %d" % tid
+            assert bool((filled == 5 + 100 * tid).all()), "fill on thread %d" % tid
+        except Exception as e:      # reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert_no_library_error(sa)
