@@ -164,6 +164,11 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch) {
     std::vector<const char*> copts;
     for (auto& o : opts) copts.push_back(o.c_str());
 
+    // One compile at a time: callers compile different ops from different threads, and nothing
+    // promises that the compiler library underneath tolerates that.
+    static std::mutex compile_mu;
+    std::lock_guard<std::mutex> compile_guard(compile_mu);
+
     hiprtcProgram prog = nullptr;
     hiprtcResult rc = hiprtcCreateProgram(&prog, source.c_str(), "sideaware_elementwise.hip",
                                           (int)(sizeof kCompatNames / sizeof *kCompatNames),

@@ -309,9 +309,12 @@ struct CompiledKernel {
 };
 
 struct KernelEntry {
-    std::string header;
+    std::string header;         // fixed at registration
+    int default_groups = 0;     // fixed at registration; 0: decide from occupancy
+    // Guards function_name and compiled[]: a first-use compile of one op (hundreds of
+    // milliseconds) does not hold up launches of the others.
+    std::mutex mu;
     std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`
-    int default_groups = 0;     // 0: decide from occupancy
     // [device * kVariants + variant]; variant = wide_index | beyond_cache << 1 | in_place << 2.
     // Fixed size: launches keep pointers into it while other threads compile other variants.
     std::array<CompiledKernel, kMaxDevices * kVariants> compiled;
@@ -363,14 +366,22 @@ static std::string full_source(const std::string& header, int variant, int num_x
 
 // Returns the compiled function for (id, variant) on ctx's device, building it on first use
 // (sideaware.cu:772-813).  Null after a failed compile; the failure is reported once.
-static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant) {
+static KernelEntry* find_entry(int kernel_id) {
     std::lock_guard<std::mutex> g(g_kernels_mu);
     ensure_builtin_locked();
     if (kernel_id < 0 || kernel_id >= (int)g_kernels.size()) {
         set_error("kernel id %d was never created", kernel_id);
         return nullptr;
     }
-    KernelEntry& e = *g_kernels[kernel_id];
+    return g_kernels[kernel_id].get();      // entries are never removed
+}
+
+static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant, KernelEntry** entry = nullptr) {
+    KernelEntry* found = find_entry(kernel_id);
+    if (entry) *entry = found;
+    if (!found) return nullptr;
+    KernelEntry& e = *found;
+    std::lock_guard<std::mutex> g(e.mu);
     if (ctx->device >= kMaxDevices) {
         set_error("device %d is beyond the %d devices this build keeps kernels for", ctx->device, kMaxDevices);
         return nullptr;
@@ -403,7 +414,7 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
         if (hipModuleGetGlobal(&name_ptr, &name_bytes, k.module, "sideaware_kernel_name") == hipSuccess &&
             name_bytes > 1 && name_bytes < sizeof name &&
             hipMemcpyDtoH(name, name_ptr, name_bytes) == hipSuccess && name[0]) {
-            e.function_name = name;               // the registry lock is held
+            e.function_name = name;               // e.mu is held
         } else {
             (void)hipGetLastError();
         }
@@ -571,14 +582,10 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     const int in_place = (!beyond && out0 != nullptr && out0 == in0) ? 4 : 0;
     const int variant = wide | beyond | in_place;
 
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant);
+    KernelEntry* entry = nullptr;
+    CompiledKernel* k = get_kernel(ctx, kernel_id, variant, &entry);
     if (!k) return;
-
-    int default_groups;
-    {
-        std::lock_guard<std::mutex> g(g_kernels_mu);
-        default_groups = g_kernels[kernel_id]->default_groups;
-    }
+    const int default_groups = entry->default_groups;
     // Workgroups per XCD.  The caller's parallel_groups / forced_per_side, or the header's
     // default, fix a persistent grid of (CUs per XCD) x groups; otherwise the tuning decides
     // between one workgroup per tile and a persistent grid sized from the kernel's occupancy.
@@ -774,13 +781,10 @@ const char* sideaware_config_block(int variant) {
 int sideaware_kernel_info(int kernel_id, int variant, int* out) {
     DeviceContext* ctx = get_context();
     if (!ctx || !out) return 1;
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & (kVariants - 1));
+    KernelEntry* entry = nullptr;
+    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & (kVariants - 1), &entry);
     if (!k) return 1;
-    int groups;
-    {
-        std::lock_guard<std::mutex> g(g_kernels_mu);
-        groups = g_kernels[kernel_id]->default_groups;
-    }
+    int groups = entry->default_groups;
     if (groups <= 0) {
         groups = k->occupancy > 0 ? k->occupancy : 4;
         if (groups > g_tune.groups_cap) groups = (int)g_tune.groups_cap;
