@@ -7,6 +7,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <ctime>
 #include <fstream>
 #include <mutex>
@@ -37,6 +38,12 @@ std::string rocm_root() {
 
 uint64_t fnv1a(const std::string& s, uint64_t h = 1469598103934665603ull) {
     for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+    return h;
+}
+
+uint64_t fnv1a(const std::vector<char>& v) {
+    uint64_t h = 1469598103934665603ull;
+    for (char c : v) { h ^= (unsigned char)c; h *= 1099511628211ull; }
     return h;
 }
 
@@ -75,6 +82,26 @@ void write_file_atomic(const std::string& path, const std::vector<char>& data) {
     if (::rename(tmp.c_str(), path.c_str()) != 0) ::unlink(tmp.c_str());
 }
 
+// A cache file is the code object followed by the eight bytes of its FNV-1a hash: a file that was
+// cut short or damaged reads as a miss instead of reaching the module loader.
+bool read_cached_code(const std::string& path, std::vector<char>& code) {
+    std::vector<char> raw;
+    if (!read_file(path, raw) || raw.size() <= 8 + 4) return false;
+    uint64_t stored = 0;
+    std::memcpy(&stored, raw.data() + raw.size() - 8, 8);
+    raw.resize(raw.size() - 8);
+    if (fnv1a(raw) != stored || std::memcmp(raw.data(), "\177ELF", 4) != 0) return false;
+    code.swap(raw);
+    return true;
+}
+
+void write_cached_code(const std::string& path, const std::vector<char>& code) {
+    std::vector<char> raw(code);
+    const uint64_t h = fnv1a(code);
+    raw.insert(raw.end(), (const char*)&h, (const char*)&h + 8);
+    write_file_atomic(path, raw);
+}
+
 void dump_isa(const std::vector<char>& code) {
     std::string file;
     {
@@ -111,7 +138,7 @@ void set_isa_dump_file(const std::string& filename) {
     g_isa_file = filename;
 }
 
-CompileResult compile_for_gfx950(const std::string& source, const char* arch) {
+CompileResult compile_for_gfx950(const std::string& source, const char* arch, bool use_disk_cache) {
     CompileResult res;
 
     char cwd_buf[4096];
@@ -153,7 +180,7 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch) {
         char name[64];
         std::snprintf(name, sizeof name, "/%016llx.co", (unsigned long long)h);
         cache_path = dir + name;
-        if (read_file(cache_path, res.code)) {
+        if (use_disk_cache && read_cached_code(cache_path, res.code)) {
             res.ok = true;
             res.from_disk_cache = true;
             dump_isa(res.code);
@@ -204,7 +231,7 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch) {
         return res;
     }
     res.ok = true;
-    if (!cache_path.empty()) write_file_atomic(cache_path, res.code);
+    if (!cache_path.empty()) write_cached_code(cache_path, res.code);
     dump_isa(res.code);
     return res;
 }

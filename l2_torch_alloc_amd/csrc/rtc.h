@@ -16,8 +16,11 @@ struct CompileResult {
 };
 
 // Compiles `source` (one translation unit, already holding the configuration block, the user's
-// header and the kernel template).  Needs no GPU: hipRTC cross-compiles.
-CompileResult compile_for_gfx950(const std::string& source, const char* arch = "gfx950");
+// header and the kernel template).  Needs no GPU: hipRTC cross-compiles.  `use_disk_cache` false
+// compiles afresh and overwrites whatever the cache holds for this source (the way out when a
+// cached code object turns out not to load).
+CompileResult compile_for_gfx950(const std::string& source, const char* arch = "gfx950",
+                                 bool use_disk_cache = true);
 
 // Where every later successful compile appends its disassembly ("" = nowhere).  The reference
 // dumps SASS through cuobjdump (sideaware.cu:572-599); here it is the gfx950 ISA of the code

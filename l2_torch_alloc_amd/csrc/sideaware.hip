@@ -405,6 +405,14 @@ static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant
     }
     ScopedDevice guard(ctx->device);
     hipError_t err = hipModuleLoadData(&k.module, r.code.data());
+    if (err != hipSuccess && r.from_disk_cache) {
+        // a cached code object the runtime refuses (damaged file, another driver): build it again
+        (void)hipGetLastError();
+        k.module = nullptr;
+        r = compile_for_gfx950(full_source(e.header, variant, ctx->num_xcds, ctx->num_cus), "gfx950",
+                               /*use_disk_cache=*/false);
+        err = r.ok ? hipModuleLoadData(&k.module, r.code.data()) : hipErrorInvalidImage;
+    }
     if (err == hipSuccess) {
         // The module itself says what its entry point is called: the header text may not (a
         // header that is only `#include "file"`, example_llmc_rope.cu:138).

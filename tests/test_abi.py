@@ -256,3 +256,26 @@ def test_a_plain_c_program_links_and_runs_against_the_header(lib, tmp_path):
     proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "c host ok" in proc.stdout
+
+
+def test_damaged_cache_files_read_as_misses(lib, tmp_path, monkeypatch):
+    # the on-disk cache of code objects: a second compile is served from it; a file that was cut
+    # short or overwritten is ignored and replaced, never handed to the module loader
+    import time
+    monkeypatch.setenv("SIDEAWARE_CACHE_DIR", str(tmp_path / "cache"))
+    header = headers.fill_header().replace(b"sideaware_fill_int32", b"sideaware_fill_cache_test")
+    t0 = time.perf_counter()
+    assert compile_ok(lib, header, 0)[0] == 0
+    cold = time.perf_counter() - t0
+    files = list((tmp_path / "cache").glob("*.co"))
+    assert len(files) == 1 and files[0].stat().st_size > 1000
+    good = files[0].read_bytes()
+    assert good[:4] == b"\x7fELF"
+    t0 = time.perf_counter()
+    assert compile_ok(lib, header, 0)[0] == 0
+    warm = time.perf_counter() - t0
+    assert warm < cold / 3, (cold, warm)                       # no compiler run the second time
+    for damaged in (good[:len(good) // 2], b"garbage" * 300, good[:-1] + bytes([good[-1] ^ 1]), b""):
+        files[0].write_bytes(damaged)
+        assert compile_ok(lib, header, 0)[0] == 0
+        assert files[0].read_bytes() == good                    # rebuilt: same source, same code object
