@@ -251,6 +251,45 @@ def bench_rope_fp32_gpt2(steps, warmup):
             "note": "25 MB: launch-bound and Infinity-Cache resident, not an HBM roofline case"}
 
 
+def bench_other_ops(steps):
+    """The other ops the framework ships, each at a size past the caches, launched through the C
+    entry point: bf16 scale+bias out of place, bf16 -> MXFP8 quantisation (a per-32 cross-lane
+    reduction with a sideband output), and fp32 RoPE forward / backward in place on the packed QKV
+    tensor of the reference's own benchmark, (8,1024,3*32,128) (example_llmc_rope.cu:247-250)."""
+    import torch
+    from l2_torch_alloc_amd import headers, ops, wrapper
+    lib, stream = _abi()
+    out = {}
+    n = 256 * MiB // 2                                                     # bf16 elements
+    x = torch.randn(n, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).cuda()
+    y = torch.empty_like(x)
+    sb = torch.tensor([1.25, -0.5], dtype=torch.float32, device="cuda")
+    kid = wrapper.sideaware_create_kernel(headers.scale_bias_bf16_header())
+    sec = time_region(lambda: lib.sideaware_elementwise(kid, 2 * n, y.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
+                                                        sb.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
+    out["scale_bias_bf16_256MiB"] = {"bytes": 4 * n, "us": sec * 1e6, "GBps": gbps(4 * n, sec)}
+    q = torch.empty(n, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(n // 32, dtype=torch.uint8, device="cuda")
+    kid = wrapper.sideaware_create_kernel(headers.mxfp8_quantize_header())
+    sec = time_region(lambda: lib.sideaware_elementwise(kid, 2 * n, q.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
+                                                        scales.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
+    nbytes = 2 * n + n + n // 32
+    out["mxfp8_quantize_256MiB_in"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
+    del x, y, q, scales
+    B, T, NH, HS = 8, 1024, 32, 128
+    qkv = torch.randn(B, T, 3 * NH, HS, generator=torch.Generator().manual_seed(7)).cuda()
+    freqs = ops.freqs_cis_table(HS, T, 10000.0, True).cuda()
+    # value heads are neither read nor written: two thirds of the tensor move, both ways
+    nbytes = 2 * (qkv.numel() * 4 * 2 // 3) + freqs.numel() * 4
+    for name, backward in (("rope_fp32_qkv_forward_llmc_shape", False), ("rope_fp32_qkv_backward_llmc_shape", True)):
+        kid = wrapper.sideaware_create_kernel(headers.rope_header(T, NH, NH, HS, "fp32", "qkv", backward=backward))
+        sec = time_region(lambda: lib.sideaware_elementwise(kid, qkv.numel() * 4, qkv.data_ptr(), 0, 0, 0,
+                                                            qkv.data_ptr(), freqs.data_ptr(), 0, 0, 0, 0, 0, 0, 0,
+                                                            stream), steps, 3)
+        out[name] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
+    return out
+
+
 def stripe_ab(steps):
     """A/B evidence for the stripe -> XCD map, meant to be run under `rocprofv3 --pmc FETCH_SIZE`:
     the q RoPE with 4 KiB tiles (half a token row), once with 4 KiB ownership stripes, so the two
@@ -458,6 +497,8 @@ def main():
             sweep[label] = bench_copy(nbytes, steps, 3, "fp32", seed=3)
             log("sweep", label, sweep[label])
         also["copy_sweep_fp32"] = sweep
+        also["other_ops"] = bench_other_ops(30)
+        log("other ops:", also["other_ops"])
         also["copy_256MiB_cold_cache"] = bench_copy_cold(256 * MiB, 20)
         also["copy_256MiB_rotating_8_pairs"] = bench_copy_rotating(256 * MiB, 8, 10)
         log("rotating:", also["copy_256MiB_rotating_8_pairs"])
