@@ -430,7 +430,43 @@ def cpu_baseline():
         L.oracle_rope_forward_heads_bf16(out.ctypes.data, x.ctypes.data, table.ctypes.data, 1, T, NH, HS)
         rt.append(time.perf_counter() - t0)
     rope_gbps = gbps(2 * x.nbytes + table.nbytes, statistics.median(rt))
+    # beside the scalar port: torch's own CPU kernels on every host thread, same data shapes
+    import torch
+    threads = torch.get_num_threads()
+    src_t = torch.randint(0, 256, (256 * MiB,), dtype=torch.uint8, generator=torch.Generator().manual_seed(0))
+    src_t.clone()
+    tt = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        src_t.clone()
+        tt.append(time.perf_counter() - t0)
+    torch_clone_gbps = gbps(2 * src_t.numel(), statistics.median(tt))
+    del src_t
+    xt = torch.from_numpy(x.view(np.int16)).view(torch.bfloat16)
+    tab = torch.from_numpy(table)
+    cos, sin = tab[:, 0::2][None, :, None, :], tab[:, 1::2][None, :, None, :]
+
+    def rope_torch():
+        xf = xt.float()
+        re, im = xf[..., 0::2], xf[..., 1::2]
+        o = torch.empty_like(xf)
+        o[..., 0::2] = re * cos - im * sin
+        o[..., 1::2] = re * sin + im * cos
+        return o.to(torch.bfloat16)
+
+    got = rope_torch()
+    agree = bool(np.array_equal(got.view(torch.int16).numpy().view(np.uint16), out))
+    tt = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        rope_torch()
+        tt.append(time.perf_counter() - t0)
+    torch_rope_gbps = gbps(2 * x.nbytes + table.nbytes, statistics.median(tt))
     return {"value": copy_gbps, "unit": "GB/s", "cores": 1, "kind": "port",
+            "torch_cpu": {"threads": threads, "clone_256MiB_GBps": torch_clone_gbps,
+                          "rope_bf16_GBps": torch_rope_gbps,
+                          "rope_equals_oracle_bit_for_bit": agree,
+                          "note": "torch.clone and torch fp32 RoPE on the same host data, all host threads"},
             "sample": "oracle_memcpy (oracle/rope_oracle.c) over the same 256 MiB uint8 buffer, one host "
                       "thread, median of 9 calls",
             "rope_bf16_GBps": rope_gbps,
