@@ -370,7 +370,10 @@ def bench_churn(use_sideaware, n_ops=10000, live_cap=64 * GiB):
     return {"ops": n_ops, "alloc_p50_us": pct(t_alloc, 0.50), "alloc_p99_us": pct(t_alloc, 0.99),
             "free_p50_us": pct(t_free, 0.50), "free_p99_us": pct(t_free, 0.99),
             "elementwise_GBps": gbps(op_bytes, op_seconds) if op_seconds else None,
-            "elementwise_samples_bytes": op_bytes}
+            "elementwise_samples_bytes": op_bytes,
+            # what the allocator held from the driver at its peak (for the pool: its own counter,
+            # reported by the caller; for PyTorch's caching allocator: its statistic)
+            "peak_reserved_bytes": None if use_sideaware else int(torch.cuda.max_memory_reserved())}
 
 
 def bench_raw_alloc_calls(n=20000):
@@ -540,8 +543,10 @@ def main():
         log("rotating:", also["copy_256MiB_rotating_8_pairs"])
         also["alloc_raw_calls"] = bench_raw_alloc_calls()
         log("raw alloc:", also["alloc_raw_calls"])
+        wrapper.library().sideaware_release_unused()      # start from an empty pool, like the child process below
         also["alloc_churn_sideaware"] = bench_churn(True)
         also["alloc_churn_sideaware"]["pool"] = wrapper.sideaware_alloc_stats()
+        also["alloc_churn_sideaware"]["peak_reserved_bytes"] = also["alloc_churn_sideaware"]["pool"]["peak_reserved"]
         log("churn (sideaware):", also["alloc_churn_sideaware"])
         wrapper.library().sideaware_release_unused()
         try:

@@ -14,7 +14,8 @@
 //          go to an exact-size LIFO reuse cache, as in the reference.  A size that is not cached
 //          is carved, best fit, from the free extents of multi-GiB arenas (a driver allocation
 //          costs hundreds of microseconds; a carve costs one), or served by a cached region at
-//          most 1/8 larger, handed out whole.  When cached plus free bytes outgrow the
+//          most 1/8 larger, handed out whole, or, failing that, from the arenas again after the
+//          whole cache was folded back into them.  When cached plus free bytes outgrow the
 //          thresholds the cache is folded back into the arenas and wholly free arenas return to
 //          the backing store; the reference's four-step out-of-memory ladder ends in null
 //          (sideaware.cu:1233-1252);
@@ -86,6 +87,7 @@ struct PoolStats {
     uint64_t arenas_acquired = 0;   // arenas for large regions and arenas for slabs
     uint64_t bytes_free_arena = 0;  // free extents inside the large regions' arenas
     uint64_t bytes_free_slab_arena = 0;  // free extents inside the slabs' arenas
+    uint64_t cache_folds = 0;       // times the reuse cache was folded back to serve a request without the driver
 };
 constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
 

@@ -86,6 +86,7 @@ POOL_STAT_FIELDS = (
     "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
     "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
     "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena",
+    "cache_folds",
 )
 
 

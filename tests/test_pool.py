@@ -26,7 +26,8 @@ GiB = 1 << 30
 FIELDS = ("large_hits", "large_misses", "small_hits", "small_carves", "slabs_acquired", "backing_acquires",
           "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
           "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
-          "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena")
+          "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena",
+          "cache_folds")
 
 
 def build_harness():
@@ -353,6 +354,39 @@ def test_carved_pages_wait_for_the_stream_that_freed_them(ph):
         pool.clear_log()
         c = pool.alloc(20 * MiB, stream=7)                        # carved from pages freed on 7 and 8: mixed
         assert c and "sync_device" in pool.log()
+    finally:
+        pool.close()
+
+
+def test_cached_regions_are_folded_back_before_the_driver_is_asked(ph):
+    pool = P(ph, arena=64 * MiB)
+    try:
+        a, b, c = pool.alloc(16 * MiB), pool.alloc(16 * MiB), pool.alloc(16 * MiB)
+        pool.free(a)
+        pool.free(b)
+        assert pool.stats()["bytes_cached_large"] == 32 * MiB
+        pool.clear_log()
+        # 30 MiB: not cached, larger than the 16 MiB free tail, no cached region within one eighth.
+        # The two cached neighbours are folded back, merge, and serve it: no driver call.
+        d = pool.alloc(30 * MiB, stream=3)
+        st = pool.stats()
+        assert d == a and pool.log() == []
+        assert st["cache_folds"] == 1 and st["backing_acquires"] == 1 and st["bytes_cached_large"] == 0
+        assert st["large_misses"] == 1 and st["large_carves"] == 3          # only the very first request was a miss
+        assert st["bytes_free_arena"] == 64 * MiB - 30 * MiB - 16 * MiB
+        # with one backing allocation per region (arena size 0) regions are never split: a miss stays a miss
+        solo = P(ph, arena=0)
+        x = solo.alloc(32 * MiB)
+        solo.free(x)
+        y = solo.alloc(20 * MiB)
+        assert y != x and solo.stats()["cache_folds"] == 0 and solo.stats()["backing_acquires"] == 2
+        solo.close()
+        # pages freed on another stream are waited for when they are carved
+        pool.free(d, stream=3)
+        pool.free(c, stream=4)
+        pool.clear_log()
+        e = pool.alloc(60 * MiB, stream=5)                                    # folds again: 30 (stream 3) + 2 + 16 (stream 4) + tail
+        assert e == a and "sync_device" in pool.log()                         # mixed streams: the device is drained
     finally:
         pool.close()
 
