@@ -587,3 +587,30 @@ def test_host_threads_compile_and_launch_concurrently(sa):
         t.join(timeout=100)
     assert not errors, errors
     assert_no_library_error(sa)
+
+
+def test_rope_bf16_2gib_tensor_uses_64_bit_indices_and_matches_its_slices(sa):
+    # (64, 4096, 32, 128) bf16 is exactly 2 GiB: the 64-bit index instantiation, all-streaming
+    # class.  RoPE treats batch rows independently, so the result must equal, bit for bit, what
+    # the 32-bit instantiation gives for each (8, 4096, 32, 128) slice on its own; one slice is
+    # also held against the oracle.
+    from l2_torch_alloc_amd import ops
+    B, T, NH, HS = 64, 4096, 32, 128
+    freqs_h = O.freqs_cis(HS, T, 500000.0)
+    freqs = torch.from_numpy(freqs_h).cuda()
+    x = torch.empty(B, T, NH, HS, dtype=torch.bfloat16, device="cuda")
+    x.view(torch.int16).copy_(((torch.arange(x.numel(), device="cuda", dtype=torch.int64) * 2654435761) >> 7)
+                              .to(torch.int16).view(B, T, NH, HS))
+    x.view(torch.int16).bitwise_and_(0x3fff)               # finite, positive bf16 patterns below 2.0
+    assert x.numel() * 2 == 2 << 30
+    whole = x.clone()
+    ops.rope_forward_heads(whole, freqs)
+    for b0 in range(0, B, 8):
+        part = x[b0:b0 + 8].clone()
+        ops.rope_forward_heads(part, freqs)
+        assert torch.equal(whole[b0:b0 + 8].view(torch.int16), part.view(torch.int16)), "slice at batch %d" % b0
+    torch.cuda.synchronize()
+    one = x[40:41].cpu()
+    want = O.rope_forward_heads_bf16(bits(one), freqs_h)
+    assert np.array_equal(bits(whole[40:41]), want)
+    assert_no_library_error(sa)
