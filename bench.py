@@ -585,6 +585,11 @@ def main():
         "also": also,
         "library_error": err or None,
     }
+    rot = also.get("copy_256MiB_rotating_8_pairs")
+    if rot:
+        # the same kernel when no operand can be cache-resident (see bench_copy_rotating)
+        result["roofline"]["operands_never_cached"] = {"achieved": rot["GBps"], "frac": rot["GBps"] / HBM_PEAK_GBPS,
+                                                       "workload": "the same copy cycling over 8 (src, dst) pairs"}
     print(json.dumps(result), flush=True)
 
 
