@@ -553,7 +553,7 @@ int sideaware_create_kernel_advanced(const char* header, bool precompile, int de
     int id = register_header(header, default_num_groups);
     if (precompile) {
         if (DeviceContext* ctx = get_context()) {
-            for (int v = 0; v < 4; v++) get_kernel(ctx, id, v);      // the in-place class compiles on first use
+            for (int v = 0; v <= 4; v++) get_kernel(ctx, id, v);     // both index widths x both size classes, and in place
         }
     }
     return id;

@@ -614,3 +614,32 @@ def test_rope_bf16_2gib_tensor_uses_64_bit_indices_and_matches_its_slices(sa):
     want = O.rope_forward_heads_bf16(bits(one), freqs_h)
     assert np.array_equal(bits(whole[40:41]), want)
     assert_no_library_error(sa)
+
+
+def test_precompiled_kernel_with_default_groups(sa):
+    # sideaware_create_kernel_advanced (sideaware.cu:1421-1458): precompile builds every
+    # instantiation up front, default_num_groups makes a persistent grid the kernel's default
+    import time
+    from l2_torch_alloc_amd import headers
+    lib = sa.library()
+    text = headers.scale_bias_bf16_header().replace(b"sideaware_scale_bias_bf16", b"sideaware_scale_bias_precompiled")
+    assert b"sideaware_scale_bias_precompiled" in text
+    kid = lib.sideaware_create_kernel_advanced(text, True, 2)
+    assert kid > 0 and lib.sideaware_create_kernel_advanced(text, False, 0) == kid
+    info = (ctypes.c_int * 4)()
+    assert lib.sideaware_kernel_info(kid, 0, info) == 0 and info[3] == 2      # default workgroups per CU
+    n = 3 * MiB + 24
+    xh = torch.randn(n, generator=torch.Generator().manual_seed(11)).to(torch.bfloat16)
+    x = xh.cuda()
+    y = torch.empty_like(x)
+    sb = torch.tensor([0.5, 3.0], dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    lib.sideaware_elementwise(kid, 2 * n, y.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, sb.data_ptr(), 0, 0, 0, 0, stream)
+    lib.sideaware_elementwise(kid, 2 * n, x.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, sb.data_ptr(), 0, 0, 0, 0, stream)
+    torch.cuda.synchronize()
+    assert time.perf_counter() - t0 < 0.05                  # out of place and in place: nothing left to compile
+    want = O.scale_bias_bf16(bits(xh), 0.5, 3.0)
+    assert np.array_equal(bits(y), want) and np.array_equal(bits(x), want)
+    assert_no_library_error(sa)
