@@ -275,6 +275,10 @@ def bench_other_ops(steps):
                                                         scales.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
     nbytes = 2 * n + n + n // 32
     out["mxfp8_quantize_256MiB_in"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
+    kid = wrapper.sideaware_create_kernel(headers.mxfp8_dequantize_header())
+    sec = time_region(lambda: lib.sideaware_elementwise(kid, 2 * n, y.data_ptr(), 0, 0, 0, q.data_ptr(), 0, 0, 0,
+                                                        scales.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
+    out["mxfp8_dequantize_256MiB_out"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
     del x, y, q, scales
     B, T, NH, HS = 8, 1024, 32, 128
     qkv = torch.randn(B, T, 3 * NH, HS, generator=torch.Generator().manual_seed(7)).cuda()

@@ -210,6 +210,41 @@ def mxfp8_quantize_header(unrolled: int | None = None) -> bytes:
     return "".join(lines).encode()
 
 
+def mxfp8_dequantize_header(unrolled: int | None = None) -> bytes:
+    """MXFP8 -> bf16: the inverse of :func:`mxfp8_quantize_header`.  in0 = E4M3 bytes, the
+    sideband pointer holds the E8M0 scale bytes (one per 32 elements), out0 = bf16
+    ``element * 2^(scale - 127)``, which is exact: an E4M3 element has four significant bits.
+    A 16-byte output vector holds 8 elements, so four neighbouring vectors share a scale byte.
+    """
+    lines = ["#define KERNEL_NAME sideaware_mxfp8_dequantize\n",
+             "typedef __bf16 o0;\ntypedef unsigned char i0;\n", _UNUSED,
+             "typedef unused o1, o2, o3, i1, i2, i3;\n"]
+    if unrolled is not None:
+        lines.append("#define UNROLLED %d\n" % unrolled)
+    lines.append("constexpr bool reverse_order = false;\n" + _evict([True]))
+    lines.append(
+        "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}\n"
+        "#define CUSTOM_VECTOR_OP\n"
+        "__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size,\n"
+        "                          o0 *out0, o1 *out1, o2 *out2, o3 *out3,\n"
+        "                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,\n"
+        "                          int* sideband_memory, int sideband_value) {\n"
+        "    const int shared_exp = (int)((const unsigned char*)sideband_memory)[vec_idx >> 2] - 127;\n"
+        "    #pragma unroll\n"
+        "    for (int i = 0; i < 8; i += 4) {\n"
+        "        int packed;\n"
+        "        __builtin_memcpy(&packed, in0 + i, 4);\n"
+        "        out0[i + 0] = (__bf16)ldexpf(__builtin_amdgcn_cvt_f32_fp8(packed, 0), shared_exp);\n"
+        "        out0[i + 1] = (__bf16)ldexpf(__builtin_amdgcn_cvt_f32_fp8(packed, 1), shared_exp);\n"
+        "        out0[i + 2] = (__bf16)ldexpf(__builtin_amdgcn_cvt_f32_fp8(packed, 2), shared_exp);\n"
+        "        out0[i + 3] = (__bf16)ldexpf(__builtin_amdgcn_cvt_f32_fp8(packed, 3), shared_exp);\n"
+        "    }\n"
+        "}\n")
+    return "".join(lines).encode()
+
+
 def fill_header() -> bytes:
     """Writes the 32-bit sideband value to every element: an output-only op (no in0)."""
     return (

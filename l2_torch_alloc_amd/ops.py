@@ -122,6 +122,19 @@ def mxfp8_quantize(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Op
     return q, scales
 
 
+def mxfp8_dequantize(q: torch.Tensor, scales: torch.Tensor, out: Optional[torch.Tensor] = None):
+    """MXFP8 -> bf16: ``q`` E4M3 bytes (uint8), ``scales`` one E8M0 byte per 32 elements."""
+    assert q.dtype == torch.uint8 and scales.dtype == torch.uint8 and q.is_contiguous() and scales.is_contiguous()
+    assert q.numel() % 32 == 0 and scales.numel() == q.numel() // 32
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+    assert out.dtype == torch.bfloat16 and out.numel() == q.numel()
+    kid = _kernel(("mxfp8_dequantize",), headers.mxfp8_dequantize_header)
+    # out0 is the wider array, so the custom op's own sizing (from out0) is the right one
+    torch.ops.sideaware.elementwise(kid, out, None, None, None, q, None, None, None, scales, 0, 0, 0)
+    return out
+
+
 def fill_int32(out: torch.Tensor, value: int):
     """Writes a 32-bit pattern over ``out`` (byte size a multiple of 16): an output-only op."""
     kid = _kernel(("fill",), headers.fill_header)

@@ -118,6 +118,7 @@ SHIPPED_HEADERS = {
     "fill": headers.fill_header(),
     "scale_bias_bf16": headers.scale_bias_bf16_header(),
     "mxfp8_quantize": headers.mxfp8_quantize_header(),
+    "mxfp8_dequantize": headers.mxfp8_dequantize_header(),
     "rope_fp32_qkv_gpt2": headers.rope_header(1024, 12, 12, 64, "fp32", "qkv"),
     "rope_fp32_heads_gpt2": headers.rope_header(1024, 12, 0, 64, "fp32", "heads"),
     "rope_fp32_qkv_ref": headers.rope_header(1024, 32, 32, 128, "fp32", "qkv"),

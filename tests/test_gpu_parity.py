@@ -350,6 +350,38 @@ def test_mxfp8_quantize_vs_oracle(sa):
     assert torch.equal(q1, q2) and torch.equal(s1, s2)
 
 
+def test_mxfp8_dequantize_vs_oracle(sa):
+    from l2_torch_alloc_amd import ops
+    gen = torch.Generator().manual_seed(18)
+    n = 32 * 30000 + 32 * 5
+    mag = torch.exp(torch.rand(n // 32, generator=gen) * 40 - 20).repeat_interleave(32)
+    xh = (torch.randn(n, generator=gen) * mag).to(torch.bfloat16)
+    q_h, s_h = O.mxfp8_quantize(bits(xh))
+    got = ops.mxfp8_dequantize(torch.from_numpy(q_h).cuda(), torch.from_numpy(s_h).cuda())
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    want = O.mxfp8_dequantize(q_h, s_h)
+    assert np.array_equal(bits(got), want)
+    # an independent route to the same numbers: torch's own float8 decoding and power of two
+    via_torch = (torch.from_numpy(q_h).view(torch.float8_e4m3fn).float() *
+                 torch.exp2(torch.from_numpy(s_h).float() - 127).repeat_interleave(32)).to(torch.bfloat16)
+    assert np.array_equal(bits(via_torch), want)
+    # every E4M3 code except the two NaNs, under scale bytes from one end of E8M0 to the other
+    # (results from bf16 subnormals up to infinity)
+    codes = np.array([c for c in range(256) if c & 0x7f != 0x7f] + [0] * 2, dtype=np.uint8)      # 256 entries
+    scale_bytes = np.array([0, 1, 9, 60, 127, 128, 200, 246, 254], dtype=np.uint8)
+    q_all = np.tile(codes, len(scale_bytes))
+    s_all = np.repeat(scale_bytes, len(codes) // 32)
+    got = ops.mxfp8_dequantize(torch.from_numpy(q_all).cuda(), torch.from_numpy(s_all).cuda())
+    torch.cuda.synchronize()
+    want = O.mxfp8_dequantize(q_all, s_all)
+    assert np.array_equal(bits(got), want)
+    # and the pair is a projection: quantise(dequantise(q, s)) == (q, s) on the quantiser's own output
+    q2, s2 = ops.mxfp8_quantize(ops.mxfp8_dequantize(torch.from_numpy(q_h).cuda(), torch.from_numpy(s_h).cuda()))
+    torch.cuda.synchronize()
+    assert np.array_equal(q2.cpu().numpy(), q_h) and np.array_equal(s2.cpu().numpy(), s_h)
+
+
 # --------------------------------------------------------------------------------------- RoPE
 
 def rel_err(got: np.ndarray, want: np.ndarray) -> float:
