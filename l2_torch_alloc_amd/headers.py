@@ -5,12 +5,12 @@ An op header is the text the caller hands to ``sideaware_create_kernel``: elemen
 hooks.  The contract is the reference's (``sideaware.cu:33-48``, ``kernel_rope.cuh:1-60``,
 ``test.py:191-216``); the generators below bake the problem shape into the text the way the
 reference's RoPE header does with its ``constexpr int T / n_head / head_dim``
-(``kernel_rope.cuh:21-27``), but for any shape, for bf16 storage and for separate q / k tensors.
+(``kernel_rope.cuh:21-27``), but for any shape, for bf16 or fp16 storage and for separate q / k tensors.
 
 Arithmetic follows the llm.c formula (``example_llmc_rope.cu:70-81``, ``kernel_rope.cuh:29-40``):
 ``out = (x_re*c - x_im*s, x_re*s + x_im*c)`` in fp32, each product rounded before the add (the
 library compiles with contraction off), so fp32 results are bit-identical to a CPU that does not
-fuse.  bf16 storage widens exactly, computes in fp32 and rounds to nearest even on store.
+fuse.  bf16 and fp16 storage widen exactly, compute in fp32 and round to nearest even on store.
 """
 from __future__ import annotations
 
@@ -40,6 +40,7 @@ _ROPE_TYPES = {
     # storage dtype -> (declarations, element type of one (re, im) pair, widen, narrow)
     "fp32": ("", "float2", "%s", "%s"),
     "bf16": ("struct sa_bf16_pair { __bf16 x, y; };\n", "sa_bf16_pair", "(float)%s", "(__bf16)(%s)"),
+    "fp16": ("struct sa_fp16_pair { _Float16 x, y; };\n", "sa_fp16_pair", "(float)%s", "(_Float16)(%s)"),
 }
 
 
@@ -59,7 +60,7 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     ``num_bytes`` at launch is the byte size of the activation tensor.
     """
     if dtype not in _ROPE_TYPES:
-        raise ValueError("dtype must be 'fp32' or 'bf16'")
+        raise ValueError("dtype must be 'fp32', 'bf16' or 'fp16'")
     if layout not in ("qkv", "heads"):
         raise ValueError("layout must be 'qkv' or 'heads'")
     if head_dim % 2:

@@ -58,8 +58,10 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
         dtype = "fp32"
     elif x.dtype == torch.bfloat16:
         dtype = "bf16"
+    elif x.dtype == torch.float16:
+        dtype = "fp16"
     else:
-        raise TypeError("RoPE storage is float32 or bfloat16")
+        raise TypeError("RoPE storage is float32, bfloat16 or float16")
     assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
     if out is None:
         out = x

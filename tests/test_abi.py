@@ -126,6 +126,7 @@ SHIPPED_HEADERS = {
     "rope_bf16_k_llama3": headers.rope_header(4096, 8, 0, 128, "bf16", "heads"),
     "rope_bf16_qkv_gqa": headers.rope_header(4096, 32, 8, 128, "bf16", "qkv"),
     "rope_fp32_backward": headers.rope_header(1024, 12, 12, 64, "fp32", "qkv", backward=True),
+    "rope_fp16_q": headers.rope_header(2048, 16, 0, 64, "fp16", "heads"),
 }
 
 

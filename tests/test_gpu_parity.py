@@ -530,9 +530,9 @@ def _random_rope_cases(count, seed):
     rng = random.Random(seed)
     cases = []
     while len(cases) < count:
-        dtype = rng.choice(["fp32", "bf16"])
+        dtype = rng.choice(["fp32", "bf16", "fp16"])
         layout = rng.choice(["qkv", "heads"])
-        head_dim = rng.choice([8, 16, 32, 64, 128, 256] if dtype == "bf16" else [4, 8, 12, 64, 96, 128])
+        head_dim = rng.choice([4, 8, 12, 64, 96, 128] if dtype == "fp32" else [8, 16, 32, 64, 128, 256])
         n_q = rng.randint(1, 8)
         n_kv = rng.randint(1, n_q) if layout == "qkv" else 0
         cases.append(dict(dtype=dtype, layout=layout, head_dim=head_dim, n_q=n_q, n_kv=n_kv,
@@ -543,14 +543,14 @@ def _random_rope_cases(count, seed):
     return cases
 
 
-@pytest.mark.parametrize("case", _random_rope_cases(16, seed=20), ids=lambda c: "%s-%s-d%d-q%d-kv%d-B%d-T%d%s%s" % (
+@pytest.mark.parametrize("case", _random_rope_cases(24, seed=20), ids=lambda c: "%s-%s-d%d-q%d-kv%d-B%d-T%d%s%s" % (
     c["dtype"], c["layout"], c["head_dim"], c["n_q"], c["n_kv"], c["B"], c["T"],
     "-bwd" if c["backward"] else "", "-inplace" if c["in_place"] else ""))
 def test_rope_random_shapes_vs_oracle(sa, case):
     # Seeded random shapes, ragged against every tile size: head counts that are not powers of two,
     # T = 1, head_dim down to one vector per head, grouped k/v heads, forward and backward, in place
-    # and out of place, both dtypes.  Bit for bit against the oracle (bf16: the oracle's fp32
-    # arithmetic on the widened inputs, narrowed round-to-nearest-even).
+    # and out of place, all three storage types.  Bit for bit against the oracle (bf16 and fp16: the
+    # oracle's fp32 arithmetic on the widened inputs, narrowed round-to-nearest-even).
     from l2_torch_alloc_amd import ops
     c = case
     heads = c["n_q"] + 2 * c["n_kv"] if c["layout"] == "qkv" else c["n_q"]
@@ -558,6 +558,8 @@ def test_rope_random_shapes_vs_oracle(sa, case):
     xh = torch.randn(c["B"], c["T"], heads, c["head_dim"], generator=gen)
     if c["dtype"] == "bf16":
         xh = xh.to(torch.bfloat16)
+    elif c["dtype"] == "fp16":
+        xh = xh.to(torch.float16)
     freqs_h = O.freqs_cis(c["head_dim"], c["T"], c["theta"], c["scaled"])
     want = _oracle_rope(xh.float().numpy(), freqs_h, c["layout"], c["n_q"], c["n_kv"], c["backward"])
     x = xh.cuda()
@@ -571,6 +573,9 @@ def test_rope_random_shapes_vs_oracle(sa, case):
     got_h = got.cpu()
     if c["dtype"] == "bf16":
         assert np.array_equal(bits(got_h[:, :, :rotated]), O.f32_to_bf16(want[:, :, :rotated]))
+    elif c["dtype"] == "fp16":
+        # IEEE round-to-nearest-even narrowing: numpy's float32 -> float16 conversion
+        assert np.array_equal(bits(got_h[:, :, :rotated]), want[:, :, :rotated].astype(np.float16).view(np.uint16))
     else:
         assert np.array_equal(bits(got_h[:, :, :rotated]), want[:, :, :rotated].view(np.uint32))
     if rotated < heads:

@@ -148,6 +148,8 @@ ROPE_SHAPES = [
     (8, 32, 0, 128, "bf16", "heads", 0),
     (6, 8, 0, 128, "bf16", "heads", 1),
     (4, 4, 2, 32, "bf16", "qkv", 1),
+    (8, 5, 0, 64, "fp16", "heads", 0),
+    (4, 4, 2, 16, "fp16", "qkv", 1),
 ]
 
 
