@@ -86,11 +86,6 @@ void Pool::note_reserved(int64_t delta) {
 // Large path
 // ---------------------------------------------------------------------------------------------
 
-namespace {
-// Tag of a free extent whose pages were last freed on more than one stream.
-void* const kMixedStreams = (void*)(uintptr_t)1;
-}  // namespace
-
 // Adds a free extent, merging it with free neighbours of the same arena.
 void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
     ExtentIndex& ix = free_[kind];
@@ -102,7 +97,7 @@ void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
     };
     auto next = ix.by_addr.lower_bound(addr);
     if (next != ix.by_addr.end() && next->second.arena == e.arena && addr + e.bytes == next->first) {
-        if (next->second.stream != e.stream) e.stream = kMixedStreams;
+        e.freed_on.merge(next->second.freed_on);
         e.bytes += next->second.bytes;
         erase_size(next->second.bytes, next->first);
         next = ix.by_addr.erase(next);
@@ -110,7 +105,7 @@ void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
     if (next != ix.by_addr.begin()) {
         auto prev = std::prev(next);
         if (prev->second.arena == e.arena && prev->first + prev->second.bytes == addr) {
-            if (prev->second.stream != e.stream) e.stream = kMixedStreams;
+            e.freed_on.merge(prev->second.freed_on);
             addr = prev->first;
             e.bytes += prev->second.bytes;
             erase_size(prev->second.bytes, prev->first);
@@ -141,18 +136,22 @@ bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* t
     return true;
 }
 
-// Best fit from the free extents of the large regions' arenas.  Pages that were freed on another
-// stream are waited for first (stream order, as for a cached region).
+// Best fit from the free extents of the large regions' arenas.  The taking stream is ordered
+// after every other stream the extent's pages were freed on (stream order, as for a cached
+// region).
 void* Pool::carve_locked(size_t rounded, void* stream) {
     uintptr_t addr;
     Extent e;
     if (!extent_take_locked(kLargeArenas, rounded, &addr, &e)) return nullptr;
-    if (e.stream == kMixedStreams) {
+    if (e.freed_on.overflow) {
         backing_->sync_device();
         st_.device_syncs++;
-    } else if (e.stream != stream && e.stream != nullptr) {
-        backing_->order_after(e.stream, stream);
-        st_.stream_syncs++;
+    } else {
+        for (int i = 0; i < e.freed_on.count; i++) {
+            if (e.freed_on.streams[i] == stream) continue;
+            backing_->order_after(e.freed_on.streams[i], stream);
+            st_.stream_syncs++;
+        }
     }
     LargeBlock blk;
     blk.ptr = (void*)addr;
@@ -186,7 +185,7 @@ bool Pool::new_arena_locked(int kind, size_t min_bytes) {
     Extent e;
     e.bytes = want;
     e.arena = arena.get();
-    e.stream = nullptr;            // never used: nothing to wait for
+    // e.freed_on stays empty: never used, nothing to wait for
     (kind == kSlabArenas ? st_.bytes_free_slab_arena : st_.bytes_free_arena) += want;
     extent_insert_locked(kind, (uintptr_t)p, e);
     arenas_.push_back(std::move(arena));
@@ -200,7 +199,7 @@ void Pool::flush_cache_locked() {
             Extent e;
             e.bytes = blk.bytes;
             e.arena = blk.arena;
-            e.stream = blk.last_stream;
+            e.freed_on.add(blk.last_stream);
             st_.bytes_free_arena += blk.bytes;
             extent_insert_locked(kLargeArenas, (uintptr_t)blk.ptr, e);
         }
@@ -456,7 +455,7 @@ size_t Pool::release_empty_slabs_locked() {
             Extent e;
             e.bytes = s->bytes;
             e.arena = s->arena;
-            e.stream = nullptr;        // the device was drained above
+            // e.freed_on stays empty: the device was drained above
             st_.bytes_free_slab_arena += s->bytes;
             extent_insert_locked(kSlabArenas, (uintptr_t)s->base, e);
         } else {

@@ -138,10 +138,29 @@ private:
         void* last_stream = nullptr;
         Arena* arena = nullptr;
     };
+    // The streams on which the pages of a free extent were last freed: work queued there may still
+    // touch them.  Empty for pages that were never handed out (or whose device has been drained
+    // since).  The null stream is a stream like any other here.  Beyond kMax distinct streams the
+    // set only remembers that it overflowed, and whoever carves from it drains the device.
+    struct StreamSet {
+        static constexpr int kMax = 4;
+        void* streams[kMax] = {nullptr, nullptr, nullptr, nullptr};
+        int count = 0;
+        bool overflow = false;
+        void add(void* stream) {
+            for (int i = 0; i < count; i++) if (streams[i] == stream) return;
+            if (count < kMax) streams[count++] = stream;
+            else overflow = true;
+        }
+        void merge(const StreamSet& other) {
+            for (int i = 0; i < other.count; i++) add(other.streams[i]);
+            overflow = overflow || other.overflow;
+        }
+    };
     struct Extent {                // a free run of pages inside an arena
         size_t bytes = 0;
         Arena* arena = nullptr;
-        void* stream = nullptr;    // the stream its memory was last freed on, or kMixedStreams
+        StreamSet freed_on;
     };
     struct Slab {
         char* base = nullptr;

@@ -214,6 +214,9 @@ def test_block_handed_to_another_stream_waits_for_the_first(sa):
     torch.cuda.synchronize()
     assert torch.equal(result, twos)                      # B's write came last
     after = sa.sideaware_alloc_stats()
-    assert after["stream_syncs"] == before["stream_syncs"] + 1
+    # the hand-over from A to B, and possibly one more when the region was first carved for A from
+    # pages that an earlier test freed on the default stream
+    assert before["stream_syncs"] + 1 <= after["stream_syncs"] <= before["stream_syncs"] + 2
+    assert after["device_syncs"] == before["device_syncs"]          # the host never waited for the device
     lib.sideaware_free_auto(q, n, 0, b.cuda_stream)
     assert sa.sideaware_last_error() == ""

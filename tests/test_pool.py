@@ -350,10 +350,29 @@ def test_carved_pages_wait_for_the_stream_that_freed_them(ph):
         b = pool.alloc(32 * MiB, stream=8)
         pool.free(a, stream=7)
         pool.free(b, stream=8)
-        pool.L.ph_set_trim(pool.h, 0, 64 * MiB)                   # every miss folds the cache back, nothing released
         pool.clear_log()
-        c = pool.alloc(20 * MiB, stream=7)                        # carved from pages freed on 7 and 8: mixed
-        assert c and "sync_device" in pool.log()
+        c = pool.alloc(20 * MiB, stream=7)                        # the cache is folded back; carved from pages freed on 7 and on 8
+        assert c and pool.log() == ["order 8 -> 7"]               # stream 7 waits for 8, not the host for the device
+        # the rest of the extent remembers both streams
+        pool.clear_log()
+        d = pool.alloc(10 * MiB, stream=9)
+        assert d and sorted(pool.log()) == ["order 7 -> 9", "order 8 -> 9"]
+        # pages freed on the null stream are waited for like any others; never-used pages are not
+        fresh = P(ph, arena=64 * MiB)
+        a0 = fresh.alloc(16 * MiB, stream=0)
+        fresh.free(a0, stream=0)
+        fresh.clear_log()
+        b0 = fresh.alloc(60 * MiB, stream=5)                      # the 16 MiB freed on stream 0 + never-used pages
+        assert b0 == a0 and fresh.log() == ["order 0 -> 5"]
+        fresh.close()
+        # more distinct streams than an extent keeps track of: the device is drained instead
+        many = P(ph, arena=64 * MiB)
+        blocks = [many.alloc(8 * MiB, stream=20 + i) for i in range(6)]
+        for i, blk in enumerate(blocks):
+            many.free(blk, stream=20 + i)
+        many.clear_log()
+        assert many.alloc(44 * MiB, stream=1) and many.log() == ["sync_device"]
+        many.close()
     finally:
         pool.close()
 
@@ -370,7 +389,7 @@ def test_cached_regions_are_folded_back_before_the_driver_is_asked(ph):
         # The two cached neighbours are folded back, merge, and serve it: no driver call.
         d = pool.alloc(30 * MiB, stream=3)
         st = pool.stats()
-        assert d == a and pool.log() == []
+        assert d == a and pool.log() == ["order 0 -> 3"]          # no driver call; freed on stream 0, taken by 3
         assert st["cache_folds"] == 1 and st["backing_acquires"] == 1 and st["bytes_cached_large"] == 0
         assert st["large_misses"] == 1 and st["large_carves"] == 3          # only the very first request was a miss
         assert st["bytes_free_arena"] == 64 * MiB - 30 * MiB - 16 * MiB
@@ -386,7 +405,8 @@ def test_cached_regions_are_folded_back_before_the_driver_is_asked(ph):
         pool.free(c, stream=4)
         pool.clear_log()
         e = pool.alloc(60 * MiB, stream=5)                                    # folds again: 30 (stream 3) + 2 + 16 (stream 4) + tail
-        assert e == a and "sync_device" in pool.log()                         # mixed streams: the device is drained
+        # (the 2 MiB left over from the first fold still carry stream 0, on which they were freed)
+        assert e == a and sorted(pool.log()) == ["order 0 -> 5", "order 3 -> 5", "order 4 -> 5"]
     finally:
         pool.close()
 
