@@ -27,7 +27,9 @@ def test_rope_header_rejects_shapes_a_vector_would_straddle():
     with pytest.raises(ValueError):
         headers.rope_header(16, 4, 4, 12, "bf16")               # 6 pairs, vectors hold 4
     with pytest.raises(ValueError):
-        headers.rope_header(16, 4, 4, 64, "fp16")
+        headers.rope_header(16, 4, 4, 12, "fp16")               # likewise
+    with pytest.raises(ValueError):
+        headers.rope_header(16, 4, 4, 64, "fp8")                # no such storage type
     with pytest.raises(ValueError):
         headers.rope_header(16, 4, 4, 64, "fp32", layout="nope")
     text = headers.rope_header(1024, 12, 12, 64, "fp32", "qkv").decode()
