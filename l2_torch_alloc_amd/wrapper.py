@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 from typing import Optional
 
 import torch
@@ -123,7 +124,12 @@ def sideaware_create_kernel(header_code: bytes) -> int:
 
 
 def sideaware_torch_side_index():
-    return _torch_side_index        # torch.uint8 tensor with one entry per CU
+    """torch.uint8 tensor with one entry per CU; before ``sideaware_init`` a one-element zero
+    tensor, as in the reference (``example_wrapper.py:29-33``)."""
+    global _torch_side_index
+    if _torch_side_index is None:
+        _torch_side_index = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    return _torch_side_index
 
 
 def sideaware_gpu_side_index():
@@ -171,6 +177,9 @@ def sideaware_init(path: str = DEFAULT_LIBRARY, install_allocator: bool = True) 
         _lib = bind(path)
     _register_ops()
     _refresh_metadata()
+    # the reference prints this line when initialisation is done (example_wrapper.py:109); here it
+    # goes to stderr so that programs with a machine-readable stdout can use the module
+    print("L2 Side Aware metadata: %s" % (_info_str,), file=sys.stderr)
 
 
 def _refresh_metadata() -> None:
