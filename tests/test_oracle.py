@@ -277,3 +277,20 @@ def test_mxfp8_error_bound_and_idempotence():
     # quantising the dequantised values changes nothing
     q2, s2 = O.mxfp8_quantize(O.mxfp8_dequantize(q, s))
     assert np.array_equal(q2, q) and np.array_equal(s2[s != 0], s[s != 0])
+
+
+def test_fp16_narrowing_used_for_fp16_rope_is_ieee_round_to_nearest_even():
+    # fp16 RoPE storage is checked on the GPU against numpy's float32 -> float16 conversion of the
+    # oracle's fp32 result.  Pin that conversion: against torch's own, and against the textbook
+    # rule on exact midpoints between neighbouring float16 values (ties go to the even mantissa).
+    import torch
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * 8,
+                        np.array([0.0, -0.0, 65504.0, 65520.0, 1e-8, 6e-8, 6.1e-5, np.inf, -np.inf], np.float32)])
+    assert np.array_equal(x.astype(np.float16).view(np.uint16),
+                          torch.from_numpy(x).to(torch.float16).view(torch.int16).numpy().view(np.uint16))
+    lo = np.arange(0x3c00, 0x3c00 + 64, dtype=np.uint16)              # 1.0 .. in float16 steps of 2^-10
+    a, b = lo.view(np.float16).astype(np.float32), (lo + 1).view(np.float16).astype(np.float32)
+    mid = (a + b) / 2                                                  # exact in float32
+    got = mid.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, np.where(lo % 2 == 0, lo, lo + 1))
