@@ -164,6 +164,36 @@ def bench_copy_rotating(nbytes, pairs, steps):
     return {"bytes": nbytes, "pairs": pairs, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec), "bit_exact": ok}
 
 
+def bench_vendor_copies(nbytes, pairs, steps):
+    """The same cycling copy done by the platform's own copy paths, for scale: PyTorch's copy_
+    kernel and the runtime's device-to-device hipMemcpyAsync, on the same kind of buffers."""
+    import ctypes
+    import torch
+    srcs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+    dsts = [torch.zeros_like(t) for t in srcs]
+
+    def torch_cycle():
+        for d, t in zip(dsts, srcs):
+            d.copy_(t)
+
+    sec_torch = time_region(torch_cycle, steps, 1) / pairs
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+    hip.hipMemcpyAsync.restype = ctypes.c_int
+    stream = torch.cuda.current_stream().cuda_stream
+    ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
+
+    def hip_cycle():
+        for d_ptr, s_ptr in ptrs:
+            rc = hip.hipMemcpyAsync(d_ptr, s_ptr, nbytes, 3, stream)       # 3 = hipMemcpyDeviceToDevice
+            assert rc == 0, rc
+
+    sec_hip = time_region(hip_cycle, steps, 1) / pairs
+    return {"bytes": nbytes, "pairs": pairs,
+            "torch_copy_": {"us": sec_torch * 1e6, "GBps": gbps(2 * nbytes, sec_torch)},
+            "hipMemcpyAsync_d2d": {"us": sec_hip * 1e6, "GBps": gbps(2 * nbytes, sec_hip)}}
+
+
 def bench_rope_bf16(steps, warmup):
     """q (8,4096,32,128) and k (8,4096,8,128) bf16 in place, fp32 table theta=5e5: one step is
     the q launch followed by the k launch."""
@@ -545,6 +575,8 @@ def main():
         also["copy_256MiB_cold_cache"] = bench_copy_cold(256 * MiB, 20)
         also["copy_256MiB_rotating_8_pairs"] = bench_copy_rotating(256 * MiB, 8, 10)
         log("rotating:", also["copy_256MiB_rotating_8_pairs"])
+        also["vendor_copies_256MiB_rotating_8_pairs"] = bench_vendor_copies(256 * MiB, 8, 10)
+        log("vendor copies:", also["vendor_copies_256MiB_rotating_8_pairs"])
         also["alloc_raw_calls"] = bench_raw_alloc_calls()
         log("raw alloc:", also["alloc_raw_calls"])
         wrapper.library().sideaware_release_unused()      # start from an empty pool, like the child process below
