@@ -245,7 +245,18 @@ def bench_rope_bf16(steps, warmup):
 
     sec_rot = time_region(cycle, max(steps // 5, 4), 1) / len(sets)
     del sets
+
+    # for scale: the same step in eager PyTorch (complex multiply in fp32, back to bf16), out of place
+    fc = torch.view_as_complex(freqs.view(T, HS // 2, 2))[None, :, None, :]
+
+    def torch_step():
+        for t in (q, k):
+            torch.view_as_real(torch.view_as_complex(t.float().view(*t.shape[:-1], HS // 2, 2)) * fc) \
+                .view(t.shape).to(torch.bfloat16)
+
+    sec_torch = time_region(torch_step, 5, 1)
     return {"bytes": total, "us": sec * 1e6, "GBps": gbps(total, sec),
+            "torch_eager_same_step": {"us": sec_torch * 1e6, "GBps_on_the_same_algorithmic_bytes": gbps(total, sec_torch)},
             "rotating_5_sets": {"us": sec_rot * 1e6, "GBps": gbps(total, sec_rot),
                                 "note": "steps cycle through five distinct (q, k) sets: no tensor is cache-resident"},
             "frac_of_peak": gbps(total, sec) / HBM_PEAK_GBPS,
