@@ -194,6 +194,69 @@ def bench_vendor_copies(nbytes, pairs, steps):
             "hipMemcpyAsync_d2d": {"us": sec_hip * 1e6, "GBps": gbps(2 * nbytes, sec_hip)}}
 
 
+def bench_energy(seconds=2.5):
+    """Board power while copying (the reference's one performance claim is about power,
+    sideaware.cu:4): 1 GiB copies cycling over four pairs for a few seconds, with this library and
+    with PyTorch's copy_, while a thread samples the GPU's hwmon power sensor.  Reports GB/s,
+    average watts and GB per joule; None where no sensor can be read."""
+    import glob
+    import threading
+    import torch
+    sensors = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average") +
+               glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+
+    def read_watts():
+        best = None
+        for path in sensors:
+            try:
+                with open(path) as f:
+                    w = int(f.read()) / 1e6
+                best = w if best is None else max(best, w)
+            except (OSError, ValueError):
+                pass
+        return best
+
+    if read_watts() is None:
+        return None
+    lib, stream = _abi()
+    n, pairs = GiB, 4
+    srcs = [torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+    dsts = [torch.zeros_like(t) for t in srcs]
+    out = {"idle_W": read_watts()}
+    for kind in ("sideaware_memcpy", "torch_copy_"):
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                w = read_watts()
+                if w is not None:
+                    samples.append(w)
+                time.sleep(0.05)
+
+        th = threading.Thread(target=sampler)
+        th.start()
+        t0, copies = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(10):
+                for d, t in zip(dsts, srcs):
+                    if kind == "sideaware_memcpy":
+                        lib.sideaware_memcpy(d.data_ptr(), t.data_ptr(), n, 0, stream)
+                    else:
+                        d.copy_(t)
+                    copies += 1
+            torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        steady = samples[len(samples) // 4:] or samples          # skip the ramp
+        watts = sum(steady) / len(steady) if steady else None
+        rate = copies * 2 * n / dt / 1e9
+        out[kind] = {"GBps": rate, "avg_W": watts, "GB_per_J": rate / watts if watts else None,
+                     "samples": len(steady)}
+        time.sleep(0.5)
+    return out
+
+
 def bench_rope_bf16(steps, warmup):
     """q (8,4096,32,128) and k (8,4096,8,128) bf16 in place, fp32 table theta=5e5: one step is
     the q launch followed by the k launch."""
@@ -581,6 +644,8 @@ def main():
             sweep[label] = bench_copy(nbytes, steps, 3, "fp32", seed=3)
             log("sweep", label, sweep[label])
         also["copy_sweep_fp32"] = sweep
+        also["energy_copy_1GiB"] = bench_energy()
+        log("energy:", also["energy_copy_1GiB"])
         also["other_ops"] = bench_other_ops(30)
         log("other ops:", also["other_ops"])
         also["copy_256MiB_cold_cache"] = bench_copy_cold(256 * MiB, 20)
