@@ -423,6 +423,62 @@ def stripe_ab(steps):
     return out
 
 
+def chain_policy(reps=6):
+    """The evidence behind the cache-policy classes: a producer launch followed at once by a consumer
+    that reads its result (this library's copy), over buffer sets that cycle so that nothing is
+    cache-resident, with the producer's stores plain or nontemporal.  Producers: a copy (not in
+    place) and the bf16 RoPE (in place), at several sizes.  Per-launch times from HIP events."""
+    import torch
+    from l2_torch_alloc_amd import headers, ops, wrapper
+    lib, stream = _abi()
+    T, HS = 4096, 128
+    freqs = ops.freqs_cis_table(HS, T, 500000.0).cuda()
+    copy_text = headers.memcpy_header().decode()
+
+    def producer_kernel(kind, stream_out, heads=32):
+        tag = "chain_%s_%s_" % (kind, "nt" if stream_out else "plain")
+        if kind == "copy":
+            text = "#define INPUT0_STREAMING 1\n#define OUTPUT_STREAMING %d\n" % stream_out + copy_text
+        else:
+            text = headers.rope_header(T, heads, 0, HS, "bf16", "heads", stream_input=True,
+                                       stream_output=bool(stream_out)).decode()
+        return wrapper.sideaware_create_kernel(text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME " + tag).encode())
+
+    def run(kind, nbytes, stream_out, heads=32):
+        kid = producer_kernel(kind, stream_out, heads)
+        sets = min(24, max(3, (1536 * MiB) // (2 * nbytes)))
+        srcs = [torch.randn(nbytes // 2, device="cuda").to(torch.bfloat16) for _ in range(sets)]
+        mids = srcs if kind == "rope" else [torch.empty_like(t) for t in srcs]
+        outs = [torch.empty_like(t) for t in srcs]
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(sets)]
+        tp = tc = 0.0
+        for rep in range(reps + 1):
+            for i in range(sets):
+                e = evs[i]
+                e[0].record()
+                lib.sideaware_elementwise(kid, nbytes, mids[i].data_ptr(), 0, 0, 0, srcs[i].data_ptr(),
+                                          freqs.data_ptr() if kind == "rope" else 0, 0, 0, 0, 0, 0, 0, 0, stream)
+                e[1].record()
+                lib.sideaware_memcpy(outs[i].data_ptr(), mids[i].data_ptr(), nbytes, 0, stream)
+                e[2].record()
+            torch.cuda.synchronize()
+            if rep:                                   # the first pass warms up
+                tp += sum(e[0].elapsed_time(e[1]) for e in evs)
+                tc += sum(e[1].elapsed_time(e[2]) for e in evs)
+        n = reps * sets
+        return {"producer_us": tp / n * 1e3, "consumer_us": tc / n * 1e3, "total_us": (tp + tc) / n * 1e3, "sets": sets}
+
+    out = {}
+    for mib in (32, 64, 128, 256):
+        for stream_out in (0, 1):
+            out["copy_%dMiB_stores_%s" % (mib, "nt" if stream_out else "plain")] = run("copy", mib * MiB, stream_out)
+    for batch in (1, 2, 4, 8):                        # (batch, 4096, 32, 128) bf16 = batch * 32 MiB
+        for stream_out in (0, 1):
+            out["rope_in_place_%dMiB_stores_%s" % (batch * 32, "nt" if stream_out else "plain")] = \
+                run("rope", batch * 32 * MiB, stream_out)
+    return out
+
+
 def churn_sizes(n_ops=10000, seed=4):
     rng = random.Random(seed)
     return [max(16, int(4096 * 2 ** (rng.random() * 17)) // 16 * 16) for _ in range(n_ops)]
@@ -595,6 +651,8 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline copy and bf16 RoPE only")
     ap.add_argument("--stripe-ab", action="store_true",
                     help="only the stripe-size A/B of the q RoPE (for a FETCH_SIZE profile)")
+    ap.add_argument("--chain-policy", action="store_true",
+                    help="only the producer -> consumer experiment behind the cache-policy classes")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -620,6 +678,9 @@ def main():
 
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": stripe_ab(args.steps)}))
+        return
+    if args.chain_policy:
+        print(json.dumps({"chain_policy": chain_policy()}))
         return
 
     copy = bench_copy(256 * MiB, args.steps, args.warmup, "uint8", seed=0)
