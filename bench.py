@@ -479,6 +479,57 @@ def chain_policy(reps=6):
     return out
 
 
+READ_ONLY_HEADER = """
+#define KERNEL_NAME sideaware_read_only_%s
+#define INPUT0_STREAMING %d
+typedef int i0;
+struct unused {};
+typedef unused o0, o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {false, false, false, false};
+__device__ void elementwise_op(size_t element_idx, int sideband, o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}
+#define CUSTOM_VECTOR_OP
+__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *out0, o1 *out1, o2 *out2, o3 *out3,
+                                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,
+                                          int* sideband_memory, int sideband_value) {
+    // the loads must not be dead code: a value that never occurs would be reported
+    if ((in0[0] ^ in0[1] ^ in0[2] ^ in0[3]) == sideband_value) sideband_memory[0] = 1;
+}
+"""
+
+
+def cache_probe():
+    """What do the caches keep of data that was only read?  A read-only op over the same buffer
+    again and again, against the same op cycling through 2 GiB, for plain and nontemporal loads."""
+    import torch
+    from l2_torch_alloc_amd import wrapper
+    lib, stream = _abi()
+    big = torch.randint(0, 255, (2 * GiB,), dtype=torch.uint8, device="cuda")
+    flag = torch.zeros(4, dtype=torch.int32, device="cuda")
+    out = {}
+    for streaming in (0, 1):
+        kid = wrapper.sideaware_create_kernel((READ_ONLY_HEADER % ("nt" if streaming else "plain", streaming)).encode())
+        for mib in (32, 64, 128, 256, 512):
+            n = mib * MiB
+            base = big.data_ptr()
+
+            def same():
+                lib.sideaware_elementwise(kid, n, 0, 0, 0, 0, base, 0, 0, 0, flag.data_ptr(), -1, 0, 0, 0, stream)
+
+            def cycle():
+                for c in range(2 * GiB // n):
+                    lib.sideaware_elementwise(kid, n, 0, 0, 0, 0, base + c * n, 0, 0, 0, flag.data_ptr(), -1, 0, 0, 0,
+                                              stream)
+
+            t_same = time_region(same, 30, 3)
+            t_cycle = time_region(cycle, 3, 1) / (2 * GiB // n)
+            out["read_%dMiB_%s" % (mib, "nt" if streaming else "plain")] = {
+                "same_buffer_GBps": gbps(n, t_same), "cycling_GBps": gbps(n, t_cycle)}
+    assert int(flag[0]) == 0          # bytes are 0..254, so four equal all-ones words cannot occur
+    return out
+
+
 def churn_sizes(n_ops=10000, seed=4):
     rng = random.Random(seed)
     return [max(16, int(4096 * 2 ** (rng.random() * 17)) // 16 * 16) for _ in range(n_ops)]
@@ -653,6 +704,8 @@ def main():
                     help="only the stripe-size A/B of the q RoPE (for a FETCH_SIZE profile)")
     ap.add_argument("--chain-policy", action="store_true",
                     help="only the producer -> consumer experiment behind the cache-policy classes")
+    ap.add_argument("--cache-probe", action="store_true",
+                    help="only the read-only probe of what the caches keep of data that was merely read")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -678,6 +731,9 @@ def main():
 
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": stripe_ab(args.steps)}))
+        return
+    if args.cache_probe:
+        print(json.dumps({"cache_probe": cache_probe()}))
         return
     if args.chain_policy:
         print(json.dumps({"chain_policy": chain_policy()}))
