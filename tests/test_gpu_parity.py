@@ -680,3 +680,40 @@ def test_precompiled_kernel_with_default_groups(sa):
     want = O.scale_bias_bf16(bits(xh), 0.5, 3.0)
     assert np.array_equal(bits(y), want) and np.array_equal(bits(x), want)
     assert_no_library_error(sa)
+
+
+INPUT_ONLY_SUM = b"""
+#define KERNEL_NAME sideaware_test_input_only_sum
+typedef int i0;
+struct unused {};
+typedef unused o0, o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ void elementwise_op(size_t element_idx, int sideband, o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}
+#define CUSTOM_VECTOR_OP
+__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *out0, o1 *out1, o2 *out2, o3 *out3,
+                                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,
+                                          int* sideband_memory, int sideband_value) {
+    atomicAdd(sideband_memory, (in0[0] + in0[1] + in0[2] + in0[3]) * sideband_value);
+    atomicAdd(sideband_memory + 1, 1);
+}
+"""
+
+
+@pytest.mark.parametrize("n_ints", [4, 1024 + 4, 5 * MiB // 4 + 12, 300 * MiB // 4])
+def test_input_only_op_with_sideband_result(sa, n_ints):
+    # No output array at all: every vector of the input is visited exactly once (the vector count
+    # and a weighted sum arrive through the sideband pointer), for a tail-only array, tiles plus a
+    # tail, and a size in the all-streaming class.
+    lib = sa.library()
+    kid = lib.sideaware_create_kernel(INPUT_ONLY_SUM)
+    x = torch.randint(-1000, 1000, (n_ints,), dtype=torch.int32, device="cuda")
+    acc = torch.zeros(4, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    lib.sideaware_elementwise(kid, 4 * n_ints, 0, 0, 0, 0, x.data_ptr(), 0, 0, 0, acc.data_ptr(), 3, 0, 0, 0, stream)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert int(acc[1]) == n_ints // 4
+    want = (3 * int(x.sum(dtype=torch.int64))) & 0xffffffff
+    assert (int(acc[0]) & 0xffffffff) == want
