@@ -220,3 +220,46 @@ def test_block_handed_to_another_stream_waits_for_the_first(sa):
     assert after["device_syncs"] == before["device_syncs"]          # the host never waited for the device
     lib.sideaware_free_auto(q, n, 0, b.cuda_stream)
     assert sa.sideaware_last_error() == ""
+
+
+def test_multi_stream_churn_keeps_contents(sa):
+    # Blocks are allocated and filled on one of four streams, then checked and freed on another
+    # (ordered by an event, as a caller must), so freed pages keep moving between streams and
+    # extents carry several of them.  A block handed out while an earlier owner's work was still
+    # queued would show up as a wrong pattern.
+    import time
+    from l2_torch_alloc_amd import headers
+    lib = sa.library()
+    rng = random.Random(12)
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    fill = lib.sideaware_create_kernel(headers.fill_header())
+    staging = torch.empty(64 * MiB, dtype=torch.uint8, device="cuda")
+    before = sa.sideaware_alloc_stats()
+    live, checked = [], 0
+    deadline = time.time() + 3.0
+    while time.time() < deadline or live:
+        if live and (time.time() >= deadline or len(live) > 100 or rng.random() < 0.45):
+            ptr, n, si, val = live.pop(rng.randrange(len(live)))
+            sj = rng.randrange(4)
+            ev = torch.cuda.Event()
+            ev.record(streams[si])
+            streams[sj].wait_event(ev)
+            with torch.cuda.stream(streams[sj]):
+                lib.sideaware_memcpy(staging.data_ptr(), ptr, n, 0, streams[sj].cuda_stream)
+                assert bool((staging[:n].view(torch.int32) == val).all()), "block %x of %d bytes" % (ptr, n)
+            checked += 1
+            lib.sideaware_free_auto(ptr, n, 0, streams[sj].cuda_stream)
+        else:
+            n = max(16, int(4096 * 2 ** (rng.random() * 14)) // 16 * 16)         # 4 KiB .. 64 MiB
+            si = rng.randrange(4)
+            ptr = lib.sideaware_malloc_auto(n, 0, streams[si].cuda_stream)
+            assert ptr
+            val = rng.randrange(1, 1 << 30)
+            for _ in range(rng.choice([1, 1, 3])):                                # keep work queued behind the host
+                lib.sideaware_elementwise(fill, n, ptr, 0, 0, 0, 0, 0, 0, 0, 0, val, 0, 0, 0, streams[si].cuda_stream)
+            live.append((ptr, n, si, val))
+    torch.cuda.synchronize()
+    after = sa.sideaware_alloc_stats()
+    assert checked > 1000
+    assert after["stream_syncs"] > before["stream_syncs"] + 100      # hand-overs happened, ordered on the device
+    assert after["failures"] == before["failures"] and sa.sideaware_last_error() == ""
