@@ -556,6 +556,33 @@ def cache_probe():
     return out
 
 
+def inflight_ab(steps):
+    """A/B for the question "would more loads in flight help?", meant to be run under
+    `rocprofv3 --pmc TCC_EA0_RDREQ_sum TCC_EA0_RDREQ_LEVEL_sum TCC_CYCLE_sum`: the 1 GiB copy (both
+    sides streaming) with 1, 2, 4 and 8 sixteen-byte loads in flight per lane.  The kernel names
+    carry UNROLLED; RDREQ_LEVEL / RDREQ is the average latency of a read request at the L2's
+    memory-side port."""
+    import torch
+    from l2_torch_alloc_amd import headers, wrapper
+    lib, stream = _abi()
+    n = GiB
+    pairs = [(torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda"), torch.empty(n, dtype=torch.uint8, device="cuda"))
+             for _ in range(2)]
+    base = headers.memcpy_header().decode()
+    out = {}
+    for unrolled in (1, 2, 4, 8):
+        text = "#define UNROLLED %d\n" % unrolled + base.replace("#define KERNEL_NAME ", "#define KERNEL_NAME unrolled%d_" % unrolled)
+        kid = wrapper.sideaware_create_kernel(text.encode())
+
+        def cycle():
+            for src, dst in pairs:
+                lib.sideaware_elementwise(kid, n, dst.data_ptr(), 0, 0, 0, src.data_ptr(), 0, 0, 0, 0, 0, 0, 0, 0, stream)
+
+        sec = time_region(cycle, steps, 2) / len(pairs)
+        out["unrolled_%d" % unrolled] = {"us": sec * 1e6, "GBps": gbps(2 * n, sec)}
+    return out
+
+
 def churn_sizes(n_ops=10000, seed=4):
     rng = random.Random(seed)
     return [max(16, int(4096 * 2 ** (rng.random() * 17)) // 16 * 16) for _ in range(n_ops)]
@@ -730,6 +757,8 @@ def main():
                     help="only the stripe-size A/B of the q RoPE (for a FETCH_SIZE profile)")
     ap.add_argument("--chain-policy", action="store_true",
                     help="only the producer -> consumer experiment behind the cache-policy classes")
+    ap.add_argument("--inflight-ab", action="store_true",
+                    help="only the 1 GiB copy with 1/2/4/8 loads in flight per lane (for a read-latency profile)")
     ap.add_argument("--cache-probe", action="store_true",
                     help="only the read-only probe of what the caches keep of data that was merely read")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
@@ -757,6 +786,9 @@ def main():
 
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": stripe_ab(args.steps)}))
+        return
+    if args.inflight_ab:
+        print(json.dumps({"inflight_ab": inflight_ab(args.steps)}))
         return
     if args.cache_probe:
         print(json.dumps({"cache_probe": cache_probe()}))
