@@ -26,9 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-MiB = 1 << 20
-GiB = 1 << 30
-HBM_PEAK_GBPS = 8000.0
+from bench_util import GiB, HBM_PEAK_GBPS, MiB, _abi, gbps, log, time_each, time_region  # noqa: E402
 
 # Bytes per launch that cross the L2 -> fabric boundary, measured with rocprofv3 --pmc (FETCH_SIZE in
 # one run, WRITE_SIZE in another, KiB per dispatch), each scaled by what the same counter reads for
@@ -39,59 +37,6 @@ COPY_256MIB_TRAFFIC_BYTES = int((131081.2 * 1.99981 + 262144.0) * 1024)       # 
 ROPE_Q_TRAFFIC_BYTES = int((132103.1 * 1.99981 + 262144.5) * 1024)            # 539.0 MB, 1.0000 x algorithmic
 ROPE_K_TRAFFIC_BYTES = int((33807.5 * 1.99981 + 65536.1) * 1024)              # 136.3 MB, 1.0002 x algorithmic
 
-
-def log(*a):
-    print(*a, file=sys.stderr, flush=True)
-
-
-# ------------------------------------------------------------------------------------- timing
-
-def time_region(fn, steps, warmup):
-    """Average seconds per call of fn over `steps` back-to-back launches on the current stream,
-    bracketed by HIP events on that stream."""
-    import torch
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        fn()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) * 1e-3 / steps
-
-
-def time_each(fn, steps, warmup, before=None):
-    """Per-launch times (seconds), each launch bracketed by its own event pair; `before` runs
-    untimed ahead of every launch (e.g. a cache flush)."""
-    import torch
-    for _ in range(warmup):
-        fn()
-    out = []
-    for _ in range(steps):
-        if before:
-            before()
-        start = torch.cuda.Event(enable_timing=True)
-        stop = torch.cuda.Event(enable_timing=True)
-        start.record()
-        fn()
-        stop.record()
-        torch.cuda.synchronize()
-        out.append(start.elapsed_time(stop) * 1e-3)
-    return out
-
-
-def gbps(nbytes, seconds):
-    return nbytes / seconds / 1e9
-
-
-def _abi():
-    """The bound library and torch's current stream handle (the stream the HIP events are on)."""
-    import torch
-    from l2_torch_alloc_amd import wrapper
-    return wrapper.library(), torch.cuda.current_stream().cuda_stream
 
 
 # ------------------------------------------------------------------------------------- workloads
@@ -424,165 +369,6 @@ def bench_other_ops(steps):
     return out
 
 
-def stripe_ab(steps):
-    """A/B evidence for the stripe -> XCD map, meant to be run under `rocprofv3 --pmc FETCH_SIZE`:
-    the q RoPE with 4 KiB tiles (half a token row), once with 4 KiB ownership stripes, so the two
-    halves of a row go to two XCDs and both L2s fetch the row's table entries, and once with 16 KiB
-    and 256 KiB stripes, where a row stays on one XCD.  Kernel names carry the stripe size."""
-    import torch
-    from l2_torch_alloc_amd import headers, ops, wrapper
-    lib, stream = _abi()
-    B, T, HS = 8, 4096, 128
-    q = torch.randn(B, T, 32, HS, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
-    freqs = ops.freqs_cis_table(HS, T, 500000.0).cuda()
-    nbytes = q.numel() * 2
-    out = {}
-    for stripe in (4096, 16384, 262144):
-        assert lib.sideaware_tune(b"stripe_bytes", stripe) == 0
-        text = headers.rope_header(T, 32, 0, HS, "bf16", "heads", unrolled=1, stream_output=True).decode()
-        text = text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME stripe%d_" % stripe)
-        kid = wrapper.sideaware_create_kernel(text.encode())
-        sec = time_region(lambda: lib.sideaware_elementwise(kid, nbytes, q.data_ptr(), 0, 0, 0, q.data_ptr(),
-                                                            freqs.data_ptr(), 0, 0, 0, 0, 0, 0, 0, stream), steps, 2)
-        out["stripe_%d" % stripe] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes + freqs.numel() * 4, sec)}
-    assert lib.sideaware_tune(b"stripe_bytes", 16384) == 0
-    return out
-
-
-def chain_policy(reps=6):
-    """The evidence behind the cache-policy classes: a producer launch followed at once by a consumer
-    that reads its result (this library's copy), over buffer sets that cycle so that nothing is
-    cache-resident, with the producer's stores plain or nontemporal.  Producers: a copy (not in
-    place) and the bf16 RoPE (in place), at several sizes.  Per-launch times from HIP events."""
-    import torch
-    from l2_torch_alloc_amd import headers, ops, wrapper
-    lib, stream = _abi()
-    T, HS = 4096, 128
-    freqs = ops.freqs_cis_table(HS, T, 500000.0).cuda()
-    copy_text = headers.memcpy_header().decode()
-
-    def producer_kernel(kind, stream_out, heads=32):
-        tag = "chain_%s_%s_" % (kind, "nt" if stream_out else "plain")
-        if kind == "copy":
-            text = "#define INPUT0_STREAMING 1\n#define OUTPUT_STREAMING %d\n" % stream_out + copy_text
-        else:
-            text = headers.rope_header(T, heads, 0, HS, "bf16", "heads", stream_input=True,
-                                       stream_output=bool(stream_out)).decode()
-        return wrapper.sideaware_create_kernel(text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME " + tag).encode())
-
-    def run(kind, nbytes, stream_out, heads=32):
-        kid = producer_kernel(kind, stream_out, heads)
-        sets = min(24, max(3, (1536 * MiB) // (2 * nbytes)))
-        srcs = [torch.randn(nbytes // 2, device="cuda").to(torch.bfloat16) for _ in range(sets)]
-        mids = srcs if kind == "rope" else [torch.empty_like(t) for t in srcs]
-        outs = [torch.empty_like(t) for t in srcs]
-        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(sets)]
-        tp = tc = 0.0
-        for rep in range(reps + 1):
-            for i in range(sets):
-                e = evs[i]
-                e[0].record()
-                lib.sideaware_elementwise(kid, nbytes, mids[i].data_ptr(), 0, 0, 0, srcs[i].data_ptr(),
-                                          freqs.data_ptr() if kind == "rope" else 0, 0, 0, 0, 0, 0, 0, 0, stream)
-                e[1].record()
-                lib.sideaware_memcpy(outs[i].data_ptr(), mids[i].data_ptr(), nbytes, 0, stream)
-                e[2].record()
-            torch.cuda.synchronize()
-            if rep:                                   # the first pass warms up
-                tp += sum(e[0].elapsed_time(e[1]) for e in evs)
-                tc += sum(e[1].elapsed_time(e[2]) for e in evs)
-        n = reps * sets
-        return {"producer_us": tp / n * 1e3, "consumer_us": tc / n * 1e3, "total_us": (tp + tc) / n * 1e3, "sets": sets}
-
-    out = {}
-    for mib in (32, 64, 128, 256):
-        for stream_out in (0, 1):
-            out["copy_%dMiB_stores_%s" % (mib, "nt" if stream_out else "plain")] = run("copy", mib * MiB, stream_out)
-    for batch in (1, 2, 4, 8):                        # (batch, 4096, 32, 128) bf16 = batch * 32 MiB
-        for stream_out in (0, 1):
-            out["rope_in_place_%dMiB_stores_%s" % (batch * 32, "nt" if stream_out else "plain")] = \
-                run("rope", batch * 32 * MiB, stream_out)
-    return out
-
-
-READ_ONLY_HEADER = """
-#define KERNEL_NAME sideaware_read_only_%s
-#define INPUT0_STREAMING %d
-typedef int i0;
-struct unused {};
-typedef unused o0, o1, o2, o3, i1, i2, i3;
-constexpr bool reverse_order = false;
-constexpr bool input_evict[4] = {false, false, false, false};
-__device__ void elementwise_op(size_t element_idx, int sideband, o0 &out0, o1 &out1, o2 &out2, o3 &out3,
-                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}
-#define CUSTOM_VECTOR_OP
-__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *out0, o1 *out1, o2 *out2, o3 *out3,
-                                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,
-                                          int* sideband_memory, int sideband_value) {
-    // the loads must not be dead code: a value that never occurs would be reported
-    if ((in0[0] ^ in0[1] ^ in0[2] ^ in0[3]) == sideband_value) sideband_memory[0] = 1;
-}
-"""
-
-
-def cache_probe():
-    """What do the caches keep of data that was only read?  A read-only op over the same buffer
-    again and again, against the same op cycling through 2 GiB, for plain and nontemporal loads."""
-    import torch
-    from l2_torch_alloc_amd import wrapper
-    lib, stream = _abi()
-    big = torch.randint(0, 255, (2 * GiB,), dtype=torch.uint8, device="cuda")
-    flag = torch.zeros(4, dtype=torch.int32, device="cuda")
-    out = {}
-    for streaming in (0, 1):
-        kid = wrapper.sideaware_create_kernel((READ_ONLY_HEADER % ("nt" if streaming else "plain", streaming)).encode())
-        for mib in (32, 64, 128, 256, 512):
-            n = mib * MiB
-            base = big.data_ptr()
-
-            def same():
-                lib.sideaware_elementwise(kid, n, 0, 0, 0, 0, base, 0, 0, 0, flag.data_ptr(), -1, 0, 0, 0, stream)
-
-            def cycle():
-                for c in range(2 * GiB // n):
-                    lib.sideaware_elementwise(kid, n, 0, 0, 0, 0, base + c * n, 0, 0, 0, flag.data_ptr(), -1, 0, 0, 0,
-                                              stream)
-
-            t_same = time_region(same, 30, 3)
-            t_cycle = time_region(cycle, 3, 1) / (2 * GiB // n)
-            out["read_%dMiB_%s" % (mib, "nt" if streaming else "plain")] = {
-                "same_buffer_GBps": gbps(n, t_same), "cycling_GBps": gbps(n, t_cycle)}
-    assert int(flag[0]) == 0          # bytes are 0..254, so four equal all-ones words cannot occur
-    return out
-
-
-def inflight_ab(steps):
-    """A/B for the question "would more loads in flight help?", meant to be run under
-    `rocprofv3 --pmc TCC_EA0_RDREQ_sum TCC_EA0_RDREQ_LEVEL_sum TCC_CYCLE_sum`: the 1 GiB copy (both
-    sides streaming) with 1, 2, 4 and 8 sixteen-byte loads in flight per lane.  The kernel names
-    carry UNROLLED; RDREQ_LEVEL / RDREQ is the average latency of a read request at the L2's
-    memory-side port."""
-    import torch
-    from l2_torch_alloc_amd import headers, wrapper
-    lib, stream = _abi()
-    n = GiB
-    pairs = [(torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda"), torch.empty(n, dtype=torch.uint8, device="cuda"))
-             for _ in range(2)]
-    base = headers.memcpy_header().decode()
-    out = {}
-    for unrolled in (1, 2, 4, 8):
-        text = "#define UNROLLED %d\n" % unrolled + base.replace("#define KERNEL_NAME ", "#define KERNEL_NAME unrolled%d_" % unrolled)
-        kid = wrapper.sideaware_create_kernel(text.encode())
-
-        def cycle():
-            for src, dst in pairs:
-                lib.sideaware_elementwise(kid, n, dst.data_ptr(), 0, 0, 0, src.data_ptr(), 0, 0, 0, 0, 0, 0, 0, 0, stream)
-
-        sec = time_region(cycle, steps, 2) / len(pairs)
-        out["unrolled_%d" % unrolled] = {"us": sec * 1e6, "GBps": gbps(2 * n, sec)}
-    return out
-
-
 def churn_sizes(n_ops=10000, seed=4):
     rng = random.Random(seed)
     return [max(16, int(4096 * 2 ** (rng.random() * 17)) // 16 * 16) for _ in range(n_ops)]
@@ -761,6 +547,12 @@ def main():
                     help="only the 1 GiB copy with 1/2/4/8 loads in flight per lane (for a read-latency profile)")
     ap.add_argument("--cache-probe", action="store_true",
                     help="only the read-only probe of what the caches keep of data that was merely read")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="only the framework-free read / write / copy kernels: what the memory system gives")
+    ap.add_argument("--launch-shapes", action="store_true",
+                    help="only the library's copy and bf16 RoPE over every ownership stripe, buffers cycling")
+    ap.add_argument("--only", action="append", default=None,
+                    help="with an experiment mode: run only the cases whose name contains this text")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -784,17 +576,24 @@ def main():
     info = wrapper.sideaware_info()
     log("device:", torch.cuda.get_device_name(0), info)
 
+    import bench_experiments as experiments
     if args.stripe_ab:
-        print(json.dumps({"stripe_ab": stripe_ab(args.steps)}))
+        print(json.dumps({"stripe_ab": experiments.stripe_ab(args.steps)}))
         return
     if args.inflight_ab:
-        print(json.dumps({"inflight_ab": inflight_ab(args.steps)}))
+        print(json.dumps({"inflight_ab": experiments.inflight_ab(args.steps)}))
         return
     if args.cache_probe:
-        print(json.dumps({"cache_probe": cache_probe()}))
+        print(json.dumps({"cache_probe": experiments.cache_probe()}))
         return
     if args.chain_policy:
-        print(json.dumps({"chain_policy": chain_policy()}))
+        print(json.dumps({"chain_policy": experiments.chain_policy()}))
+        return
+    if args.launch_shapes:
+        print(json.dumps({"launch_shapes": experiments.launch_shapes(args.steps, only=args.only)}))
+        return
+    if args.ceiling:
+        print(json.dumps({"ceiling": experiments.ceiling(args.steps, only=args.only)}))
         return
 
     copy = bench_copy(256 * MiB, args.steps, args.warmup, "uint8", seed=0)

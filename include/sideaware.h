@@ -103,6 +103,24 @@ int sideaware_hash_mask(void);
 
 /* ---- additions (no counterpart in the reference) ---------------------------------------- */
 
+/* One array of a batched launch: the same fields sideaware_elementwise takes for its one array. */
+typedef struct sideaware_segment {
+    size_t num_bytes;          /* of the array whose elements are the wider of (i0, o0) */
+    void* out[4];
+    const void* in[4];
+    void* sideband_memory;
+    int sideband_value;
+} sideaware_segment;
+/* Runs one op over several arrays in a single launch: the grid's workgroups are divided between
+ * the segments, each of which is processed exactly as sideaware_elementwise would process it
+ * (same ownership stripes, same tail handling).  Small arrays share one launch instead of paying
+ * for one each: the Llama-3 k tensor rides along with q.  All segments run the same compiled
+ * instantiation: 64-bit indices if any segment needs them, the streaming cache class if the
+ * segments together exceed the Infinity Cache, in place only if every segment is.  Segments with
+ * num_bytes 0 are skipped; more than 8 segments go out as several launches. */
+void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideaware_segment* segments,
+                                 int device, sideaware_stream_t stream);
+
 /* Upper bound on the device bytes the pool may hold (0 = none): a request that would pass it is
  * answered like one the device refused (caches are given back, then null). */
 void sideaware_reserve_limit(size_t bytes);
@@ -118,7 +136,8 @@ void sideaware_clear_error(void);
 /* Compiles header + template for gfx950 without touching a device. variant bit 0: 0 = 32-bit indices
  * (arrays below 2 GiB), 1 = 64-bit indices; bit 1: 0 = the array fits the Infinity Cache
  * (outputs written plainly), 1 = larger (everything streams); bit 2: 1 = o0 is written over i0
- * (in place: outputs stream when i0 is marked input_evict).  Returns 0 on success; the compiler
+ * (in place: outputs stream when i0 is marked input_evict); bit 3: 1 = i0 or o0 is not 2 MiB-aligned
+ * (`aligned_2MiB` is false, as it is with 64-bit indices).  Returns 0 on success; the compiler
  * log (possibly empty) is copied to `log`. */
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity);
 /* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */
@@ -131,8 +150,9 @@ const char* sideaware_config_block(int variant);
 int sideaware_kernel_info(int kernel_id, int variant, int* out);
 /* Pool counters, in the order of struct PoolStats (pool.h); returns the number written. */
 int sideaware_alloc_stats(unsigned long long* out, int capacity);
-/* Tuning knobs: "stripe_bytes", "slot_run", "groups_cap", "one_shot", "cache_bytes" (launch parameters) and
- * "nt_store", "wg_threads" (compiled in: setting one drops every compiled kernel).
+/* Tuning knobs: "stripe_bytes" (0 = chosen by array size), "stripes_per_xcd", "slot_run", "groups_cap",
+ * "one_shot", "cache_bytes" (launch parameters) and "nt_store", "wg_threads" (compiled in: after a
+ * change every op is compiled afresh on its next launch).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -1,0 +1,214 @@
+// hbm_ceiling.so: framework-free streaming kernels for gfx950 that measure what the memory system of
+// an MI355X delivers to the simplest possible read, write and copy loops.  They share nothing with
+// the elementwise template (no op hooks, no launch planner): `bench.py --ceiling` times them beside
+// the library's own kernels so that "the hardware tops out here" is a measurement, not a claim.
+//
+// Every kernel moves 16-byte vectors; a wave instruction covers 1 KiB of consecutive addresses
+// unless the lane-contiguous flag is set.  Sizes must be whole numbers of tiles: the host checks.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+enum : int {
+    kNtLoads = 1,          // loads carry the nontemporal hint
+    kNtStores = 2,         // stores carry the nontemporal hint
+    kLaneContiguous = 4,   // a lane takes K consecutive vectors instead of K vectors a block apart
+    kWaitStores = 8,       // persistent kernels: stores are acknowledged before the next loads are issued
+    kSplitRoles = 16,      // tile kernel: workgroup pairs alternate between reading src and filling dst
+};
+
+template <bool NT>
+__device__ __forceinline__ v4i ld(const v4i* p) {
+    return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st(v4i* p, v4i v) {
+    if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
+__device__ __forceinline__ void sink_if_magic(v4i acc, int* sink) {
+    // keeps the loads alive: the data is random, so four equal words of this value never occur
+    if ((acc.x ^ acc.y) == 0x5a5a5a5a && (acc.z ^ acc.w) == 0x5a5a5a5a && acc.x == acc.z) sink[0] = 1;
+}
+
+// XCD-striped tile number of a workgroup: workgroups are dealt to the 8 XCDs in turn, so the
+// workgroup with index b runs on XCD b % 8; stripe s (2^r tiles) of the array goes to XCD s % 8.
+__device__ __forceinline__ long long striped_tile(unsigned b, unsigned r) {
+    const unsigned xcd = b & 7u, slot = b >> 3;
+    return ((((long long)(slot >> r) << 3) + xcd) << r) + (slot & ((1u << r) - 1u));
+}
+
+// One workgroup per tile of K * blockDim.x vectors.  dst == nullptr: read only; src == nullptr:
+// write only; both: copy (dst == src: read-modify-write in place).
+template <int K, bool NTL, bool NTS, bool CONTIG>
+__global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, unsigned r, int flags, int* sink) {
+    const unsigned B = blockDim.x, tid = threadIdx.x;
+    const long long tile = striped_tile(blockIdx.x, r);
+    const long long base = tile * (long long)(B * K);
+    bool do_read = src != nullptr, do_write = dst != nullptr;
+    if (flags & kSplitRoles) {
+        // independent streams: half of the workgroups only read, the other half only write
+        const bool reader = ((blockIdx.x >> 3) & 1u) == 0;
+        do_read = reader;
+        do_write = !reader;
+    }
+    v4i v[K];
+    if (do_read) {
+        #pragma unroll
+        for (int k = 0; k < K; k++) {
+            const long long i = CONTIG ? base + (long long)tid * K + k : base + (long long)k * B + tid;
+            v[k] = ld<NTL>(src + i);
+        }
+    } else {
+        #pragma unroll
+        for (int k = 0; k < K; k++) v[k] = (v4i){(int)tid, k, (int)blockIdx.x, 7};
+    }
+    if (do_write) {
+        #pragma unroll
+        for (int k = 0; k < K; k++) {
+            const long long i = CONTIG ? base + (long long)tid * K + k : base + (long long)k * B + tid;
+            st<NTS>(dst + i, v[k]);
+        }
+    } else {
+        v4i acc = v[0];
+        #pragma unroll
+        for (int k = 1; k < K; k++) acc ^= v[k];
+        sink_if_magic(acc, sink);
+    }
+}
+
+// A fixed grid; workgroup b takes chunks b, b + grid, b + 2 grid, ... of K * blockDim.x vectors
+// (dst == nullptr: read only; src == nullptr: write only).
+// All K loads of a chunk are complete before its first store is issued, so each workgroup
+// alternates between a read burst and a write burst.  With period_ticks != 0 every wave waits for
+// the next multiple of period_ticks of the device's 100 MHz constant clock before each read
+// burst: the bursts of all workgroups of the chip then line up, and the memory sees alternating
+// read-mostly and write-mostly phases instead of a steady mix.
+template <int K, bool NTL, bool NTS>
+__global__ __launch_bounds__(1024) void persistent_kernel(v4i* dst, const v4i* src, long long n_chunks, int flags,
+                                                          unsigned period_ticks, int* sink) {
+    const unsigned B = blockDim.x, tid = threadIdx.x;
+    const long long chunk = (long long)B * K;
+    for (long long c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        if (period_ticks) {
+            const unsigned long long t = wall_clock64();
+            const unsigned long long target = (t / period_ticks + 1) * period_ticks;
+            while (wall_clock64() < target) __builtin_amdgcn_s_sleep(2);
+        }
+        const long long base = c * chunk + tid;
+        v4i v[K];
+        if (src) {
+            #pragma unroll
+            for (int k = 0; k < K; k++) v[k] = ld<NTL>(src + base + (long long)k * B);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            #pragma unroll
+            for (int k = 0; k < K; k++) v[k] = (v4i){(int)tid, k, (int)c, 7};
+        }
+        if (dst) {
+            #pragma unroll
+            for (int k = 0; k < K; k++) st<NTS>(dst + base + (long long)k * B, v[k]);
+            if (flags & kWaitStores) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            v4i acc = v[0];
+            #pragma unroll
+            for (int k = 1; k < K; k++) acc ^= v[k];
+            sink_if_magic(acc, sink);
+        }
+    }
+}
+
+typedef void (*tile_fn)(v4i*, const v4i*, unsigned, int, int*);
+typedef void (*persistent_fn)(v4i*, const v4i*, long long, int, unsigned, int*);
+
+template <int K>
+static tile_fn pick_tile(int flags) {
+    const bool c = flags & kLaneContiguous;
+    switch (flags & 3) {
+        case 0: return c ? tile_kernel<K, false, false, true> : tile_kernel<K, false, false, false>;
+        case 1: return c ? tile_kernel<K, true, false, true> : tile_kernel<K, true, false, false>;
+        case 2: return c ? tile_kernel<K, false, true, true> : tile_kernel<K, false, true, false>;
+        default: return c ? tile_kernel<K, true, true, true> : tile_kernel<K, true, true, false>;
+    }
+}
+
+template <int K>
+static persistent_fn pick_persistent(int flags) {
+    switch (flags & 3) {
+        case 0: return persistent_kernel<K, false, false>;
+        case 1: return persistent_kernel<K, true, false>;
+        case 2: return persistent_kernel<K, false, true>;
+        default: return persistent_kernel<K, true, true>;
+    }
+}
+
+static char g_error[256] = "";
+
+static int fail(const char* what) {
+    std::snprintf(g_error, sizeof g_error, "%s", what);
+    return 1;
+}
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+const char* hbm_ceiling_last_error(void) { return g_error; }
+
+// One workgroup per tile.  `bytes` must be a multiple of 8 * (k * block * 16) << stripe_log2.
+// Returns 0 when the kernel was launched.
+int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block, int stripe_log2, int flags,
+                     int* sink, hipStream_t stream) {
+    if (block < 64 || block > 1024 || (block & (block - 1))) return fail("block must be a power of two in 64..1024");
+    if (stripe_log2 < 0 || stripe_log2 > 12) return fail("stripe_log2 must be in 0..12");
+    if (!dst && !src) return fail("nothing to do");
+    if (!sink) return fail("sink must point at four bytes of device memory");
+    const size_t tile_bytes = (size_t)k * block * 16;
+    const size_t period = (tile_bytes * 8) << stripe_log2;
+    if (bytes == 0 || bytes % period) return fail("bytes must be a whole number of 8-XCD stripe periods");
+    const size_t tiles = bytes / tile_bytes;
+    if (tiles > 0x7fffffffull) return fail("too many tiles for one grid");
+    tile_fn fn = nullptr;
+    switch (k) {
+        case 1: fn = pick_tile<1>(flags); break;
+        case 2: fn = pick_tile<2>(flags); break;
+        case 4: fn = pick_tile<4>(flags); break;
+        case 8: fn = pick_tile<8>(flags); break;
+        case 16: fn = pick_tile<16>(flags); break;
+        default: return fail("k must be 1, 2, 4, 8 or 16");
+    }
+    hipLaunchKernelGGL(fn, dim3((unsigned)tiles), dim3(block), 0, stream, (v4i*)dst, (const v4i*)src,
+                       (unsigned)stripe_log2, flags, sink);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
+}
+
+// A fixed grid of `grid` workgroups.  `bytes` must be a multiple of k * block * 16.
+int hbm_ceiling_persistent(void* dst, const void* src, size_t bytes, int k, int block, int grid, int flags,
+                           unsigned period_ticks, int* sink, hipStream_t stream) {
+    if (block < 64 || block > 1024 || (block & (block - 1))) return fail("block must be a power of two in 64..1024");
+    if (grid < 1 || grid > (1 << 20)) return fail("grid out of range");
+    if (!dst && !src) return fail("nothing to do");
+    if (!sink) return fail("sink must point at four bytes of device memory");
+    const size_t chunk_bytes = (size_t)k * block * 16;
+    if (bytes == 0 || bytes % chunk_bytes) return fail("bytes must be a whole number of chunks");
+    persistent_fn fn = nullptr;
+    switch (k) {
+        case 1: fn = pick_persistent<1>(flags); break;
+        case 2: fn = pick_persistent<2>(flags); break;
+        case 4: fn = pick_persistent<4>(flags); break;
+        case 8: fn = pick_persistent<8>(flags); break;
+        case 16: fn = pick_persistent<16>(flags); break;
+        case 24: fn = pick_persistent<24>(flags); break;
+        default: return fail("k must be 1, 2, 4, 8, 16 or 24");
+    }
+    hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(block), 0, stream, (v4i*)dst, (const v4i*)src,
+                       (long long)(bytes / chunk_bytes), flags, period_ticks, sink);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

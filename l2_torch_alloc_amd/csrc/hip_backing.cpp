@@ -90,10 +90,17 @@ void HipBacking::order_after(void* producer, void* consumer) {
     }
 }
 
+// A pointer the pool never handed out is released by the runtime behind the work already queued
+// on `stream`, as the reference does with cudaFreeAsync (sideaware.cu:1258-1260).  Memory that did
+// not come from the runtime's stream-ordered allocator may be refused there: then the stream is
+// drained and the blocking free takes it.
 int HipBacking::free_foreign(void* ptr, void* stream) {
     DeviceGuard g(device_);
-    (void)stream;
-    hipError_t e = hipFree(ptr);
+    hipError_t e = hipFreeAsync(ptr, (hipStream_t)stream);
+    if (e == hipSuccess) return 0;
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize((hipStream_t)stream);
+    e = hipFree(ptr);
     if (e != hipSuccess) (void)hipGetLastError();
     return (int)e;
 }

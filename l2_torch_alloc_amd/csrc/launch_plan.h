@@ -52,7 +52,10 @@ inline LaunchPlan plan_launch(uint64_t base_address, long long num_vectors, int 
     p.slots = (unsigned int)slots;
     p.grid = p.slots * (unsigned int)num_xcds;
 
-    p.run = slot_run > 0 ? slot_run : (p.u_count + slots - 1) / slots;
+    // A run longer than a workgroup's whole share is the same as the share (and keeps
+    // slots * run within twice u_count, so the kernel's 32-bit stepping cannot overflow).
+    const long long share = (p.u_count + slots - 1) / slots;
+    p.run = slot_run > 0 && slot_run < share ? slot_run : share;
     if (p.run < 1) p.run = 1;
 
     if (p.full_tiles * tile_vectors < num_vectors) {

@@ -501,6 +501,7 @@ int Pool::deallocate(void* ptr, void* stream) {
         size_t off = (char*)ptr - slab->base;
         size_t idx = off / slab->block;
         if (off % slab->block != 0 || idx >= slab->carved || !slab->in_use[idx]) {
+            st_.refused_frees++;
             std::fprintf(stderr, "sideaware: free of %p, which is not a live block of this pool\n", ptr);
             return 1;
         }
@@ -510,6 +511,18 @@ int Pool::deallocate(void* ptr, void* stream) {
         st_.bytes_cached_small += slab->block;
         small_[small_class_index(slab->block)].free.push_back({ptr, stream});
         return 0;
+    }
+
+    // An address inside one of the pool's own arenas that is not a live block: a second free of a
+    // large region, an interior pointer, a pointer into free pages.  The runtime must never see
+    // it: an arena's first region starts at the arena's base, and the runtime's free of that
+    // address would take the whole arena away from under every block carved from it.
+    for (const auto& a : arenas_) {
+        if ((char*)ptr >= a->base && (char*)ptr < a->base + a->bytes) {
+            st_.refused_frees++;
+            std::fprintf(stderr, "sideaware: free of %p, which is not a live block of this pool\n", ptr);
+            return 1;
+        }
     }
 
     // Not ours (sideaware.cu:1258-1260 forwards unknown pointers to cudaFreeAsync).

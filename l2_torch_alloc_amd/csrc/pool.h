@@ -88,6 +88,7 @@ struct PoolStats {
     uint64_t bytes_free_arena = 0;  // free extents inside the large regions' arenas
     uint64_t bytes_free_slab_arena = 0;  // free extents inside the slabs' arenas
     uint64_t cache_folds = 0;       // times the reuse cache was folded back to serve a request without the driver
+    uint64_t refused_frees = 0;     // frees of addresses inside the pool that are not live blocks (double frees, interior pointers)
 };
 constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
 

@@ -1,5 +1,7 @@
 #include "rtc.h"
 
+#include <elf.h>
+#include <hip/hip_version.h>
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -45,6 +47,49 @@ uint64_t fnv1a(const std::vector<char>& v) {
     uint64_t h = 1469598103934665603ull;
     for (char c : v) { h ^= (unsigned char)c; h *= 1099511628211ull; }
     return h;
+}
+
+// True when every #include of the text names one of the in-memory compatibility headers or a
+// header below hip/ : files whose content is fixed by the ROCm installation, which the cache key
+// identifies.  Any other include (in either spelling, with any spacing) may change under the key.
+bool includes_only_toolchain_headers(const std::string& source) {
+    size_t pos = 0;
+    while ((pos = source.find('#', pos)) != std::string::npos) {
+        // a directive starts its line (blanks aside); a '#' anywhere else is text
+        size_t line = pos;
+        while (line > 0 && (source[line - 1] == ' ' || source[line - 1] == '\t')) line--;
+        const bool directive = line == 0 || source[line - 1] == '\n';
+        size_t p = pos + 1;
+        pos = p;
+        if (!directive) continue;
+        while (p < source.size() && (source[p] == ' ' || source[p] == '\t')) p++;
+        if (source.compare(p, 7, "include") != 0) continue;
+        p += 7;
+        while (p < source.size() && (source[p] == ' ' || source[p] == '\t')) p++;
+        if (p >= source.size() || (source[p] != '"' && source[p] != '<')) return false;    // a macro-built name
+        const char close = source[p] == '"' ? '"' : '>';
+        const size_t end = source.find(close, p + 1);
+        if (end == std::string::npos) return false;
+        const std::string name = source.substr(p + 1, end - p - 1);
+        bool known = name.compare(0, 4, "hip/") == 0;
+        for (const char* compat : kCompatNames) known = known || name == compat;
+        if (!known) return false;
+    }
+    return true;
+}
+
+// Names the compiler and its headers: the hipRTC version, the HIP version this library was built
+// against, and the version file of the ROCm installation the headers come from.
+std::string toolchain_identity() {
+    int maj = 0, min = 0;
+    hiprtcVersion(&maj, &min);
+    std::string id = "hiprtc " + std::to_string(maj) + "." + std::to_string(min) + " hip " +
+                     std::to_string(HIP_VERSION_MAJOR) + "." + std::to_string(HIP_VERSION_MINOR) + "." +
+                     std::to_string(HIP_VERSION_PATCH) + " rocm ";
+    std::ifstream f(rocm_root() + "/.info/version");
+    std::string line;
+    if (f && std::getline(f, line)) id += line;
+    return id;
 }
 
 std::string cache_dir() {
@@ -133,6 +178,44 @@ void dump_isa(const std::vector<char>& code) {
 
 }  // namespace
 
+size_t read_code_object_symbol(const std::vector<char>& code, const char* name, void* out, size_t capacity) {
+    const size_t size = code.size();
+    const char* base = code.data();
+    if (size < sizeof(Elf64_Ehdr) || std::memcmp(base, ELFMAG, SELFMAG) != 0 || base[EI_CLASS] != ELFCLASS64) return 0;
+    Elf64_Ehdr eh;
+    std::memcpy(&eh, base, sizeof eh);
+    if (eh.e_shentsize != sizeof(Elf64_Shdr) || eh.e_shoff > size ||
+        (size - eh.e_shoff) / sizeof(Elf64_Shdr) < eh.e_shnum) return 0;
+    auto section = [&](unsigned i, Elf64_Shdr* sh) {
+        if (i >= eh.e_shnum) return false;
+        std::memcpy(sh, base + eh.e_shoff + (size_t)i * sizeof(Elf64_Shdr), sizeof *sh);
+        return sh->sh_type == SHT_NOBITS || (sh->sh_offset <= size && sh->sh_size <= size - sh->sh_offset);
+    };
+    const size_t name_len = std::strlen(name);
+    for (unsigned i = 0; i < eh.e_shnum; i++) {
+        Elf64_Shdr symtab, strtab;
+        if (!section(i, &symtab) || (symtab.sh_type != SHT_SYMTAB && symtab.sh_type != SHT_DYNSYM)) continue;
+        if (symtab.sh_entsize != sizeof(Elf64_Sym) || !section(symtab.sh_link, &strtab) || strtab.sh_type != SHT_STRTAB) continue;
+        for (size_t k = 0; k < symtab.sh_size / sizeof(Elf64_Sym); k++) {
+            Elf64_Sym sym;
+            std::memcpy(&sym, base + symtab.sh_offset + k * sizeof sym, sizeof sym);
+            if (sym.st_name >= strtab.sh_size || strtab.sh_size - sym.st_name <= name_len) continue;
+            const char* s = base + strtab.sh_offset + sym.st_name;
+            if (std::memcmp(s, name, name_len) != 0 || s[name_len] != '\0') continue;
+            Elf64_Shdr data;
+            if (sym.st_shndx == SHN_UNDEF || sym.st_shndx >= SHN_LORESERVE || !section(sym.st_shndx, &data) ||
+                data.sh_type == SHT_NOBITS || sym.st_value < data.sh_addr) continue;
+            const uint64_t off = sym.st_value - data.sh_addr;
+            if (off > data.sh_size) continue;
+            size_t n = sym.st_size < capacity ? (size_t)sym.st_size : capacity;
+            if (n > data.sh_size - off) n = (size_t)(data.sh_size - off);
+            std::memcpy(out, base + data.sh_offset + off, n);
+            return n;
+        }
+    }
+    return 0;
+}
+
 void set_isa_dump_file(const std::string& filename) {
     std::lock_guard<std::mutex> g(g_rtc_mu);
     g_isa_file = filename;
@@ -168,15 +251,14 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch, bo
     }
 
     // Disk cache: the key covers the whole translation unit, every option and the compiler.
-    // Sources that include files by path are not cached (their content is not in the key).
-    std::string dir = source.find("#include \"") == std::string::npos ? cache_dir() : "";
+    // Sources that include anything but the ROCm headers are not cached (the content of a user's
+    // file is not in the key).
+    std::string dir = includes_only_toolchain_headers(source) ? cache_dir() : "";
     std::string cache_path;
     if (!dir.empty()) {
-        int maj = 0, min = 0;
-        hiprtcVersion(&maj, &min);
         uint64_t h = fnv1a(source);
         for (auto& o : opts) h = fnv1a(o, h);
-        h = fnv1a(std::to_string(maj) + "." + std::to_string(min), h);
+        h = fnv1a(toolchain_identity(), h);
         char name[64];
         std::snprintf(name, sizeof name, "/%016llx.co", (unsigned long long)h);
         cache_path = dir + name;

@@ -22,6 +22,12 @@ struct CompileResult {
 CompileResult compile_for_gfx950(const std::string& source, const char* arch = "gfx950",
                                  bool use_disk_cache = true);
 
+// Copies the initial bytes of a global variable out of a code object (an ELF image), on the host:
+// what a kernel says about itself (tile size, entry point name) is known without asking the
+// device, so a first-use compile neither copies from the device nor waits for it.  Returns the
+// number of bytes copied (at most `capacity`), 0 if the symbol is not there.
+size_t read_code_object_symbol(const std::vector<char>& code, const char* name, void* out, size_t capacity);
+
 // Where every later successful compile appends its disassembly ("" = nowhere).  The reference
 // dumps SASS through cuobjdump (sideaware.cu:572-599); here it is the gfx950 ISA of the code
 // object just built, through the ROCm llvm-objdump.

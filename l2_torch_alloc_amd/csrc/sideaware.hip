@@ -75,16 +75,28 @@ static void set_error(const char* fmt, ...) {
 // Tuning
 // ---------------------------------------------------------------------------------------------
 
+// A snapshot of the knobs, taken once per launch.
 struct Tuning {
-    long long stripe_bytes = 16384;  // ownership stripe of an XCD (power of two; shrunk for small arrays)
+    long long stripe_bytes = 0;      // ownership stripe of an XCD (power of two; shrunk for small arrays); 0: by array size
     long long slot_run = 1;          // tiles a workgroup takes in a row; 0 = one contiguous block each
     long long one_shot = 1;          // 1: one workgroup per tile unless the caller fixes the groups
     long long cache_bytes = 256ll << 20;   // arrays larger than this are compiled to stream in both directions
     long long nt_store = 2;          // nontemporal stores: 0 never, 1 always, 2 only for arrays beyond the Infinity Cache
     long long groups_cap = 8;        // upper bound on default workgroups per CU
     long long wg_threads = 256;
+    long long stripes_per_xcd = 8;   // an array gets stripes small enough for every XCD to own at least this many
 };
-static Tuning g_tune;
+
+// The knobs themselves: written by sideaware_tune (and once from the environment), read by every
+// launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
+// a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
+constexpr int kTuneKnobs = 8;
+static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
+                                                   "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd"};
+static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
+                                                 "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
+                                                 "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -96,26 +108,45 @@ static long long env_ll(const char* name, long long fallback) {
 static void load_tuning_from_env_once() {
     static std::once_flag once;
     std::call_once(once, [] {
-        g_tune.stripe_bytes = env_ll("SIDEAWARE_STRIPE_BYTES", g_tune.stripe_bytes);
-        g_tune.slot_run = env_ll("SIDEAWARE_SLOT_RUN", g_tune.slot_run);
-        g_tune.one_shot = env_ll("SIDEAWARE_ONE_SHOT", g_tune.one_shot);
-        g_tune.cache_bytes = env_ll("SIDEAWARE_CACHE_BYTES", g_tune.cache_bytes);
-        g_tune.nt_store = env_ll("SIDEAWARE_NT_STORE", g_tune.nt_store);
-        g_tune.groups_cap = env_ll("SIDEAWARE_GROUPS_CAP", g_tune.groups_cap);
-        g_tune.wg_threads = env_ll("SIDEAWARE_WG_THREADS", g_tune.wg_threads);
+        for (int i = 0; i < kTuneKnobs; i++) g_tune[i].store(env_ll(kTuneEnv[i], g_tune[i].load()));
     });
 }
 
-static long long* tune_slot(const char* key) {
+static Tuning tuning_snapshot() {
+    Tuning t;
+    t.stripe_bytes = g_tune[0].load(std::memory_order_relaxed);
+    t.slot_run = g_tune[1].load(std::memory_order_relaxed);
+    t.one_shot = g_tune[2].load(std::memory_order_relaxed);
+    t.cache_bytes = g_tune[3].load(std::memory_order_relaxed);
+    t.nt_store = g_tune[4].load(std::memory_order_relaxed);
+    t.groups_cap = g_tune[5].load(std::memory_order_relaxed);
+    t.wg_threads = g_tune[6].load(std::memory_order_relaxed);
+    t.stripes_per_xcd = g_tune[7].load(std::memory_order_relaxed);
+    return t;
+}
+
+static std::atomic<long long>* tune_slot(const char* key) {
     if (!key) return nullptr;
-    if (!std::strcmp(key, "stripe_bytes")) return &g_tune.stripe_bytes;
-    if (!std::strcmp(key, "slot_run")) return &g_tune.slot_run;
-    if (!std::strcmp(key, "one_shot")) return &g_tune.one_shot;
-    if (!std::strcmp(key, "cache_bytes")) return &g_tune.cache_bytes;
-    if (!std::strcmp(key, "nt_store")) return &g_tune.nt_store;
-    if (!std::strcmp(key, "groups_cap")) return &g_tune.groups_cap;
-    if (!std::strcmp(key, "wg_threads")) return &g_tune.wg_threads;
+    for (int i = 0; i < kTuneKnobs; i++) if (!std::strcmp(key, kTuneNames[i])) return &g_tune[i];
     return nullptr;
+}
+
+// The ownership stripe for an array of num_bytes.  Measured on MI355X with buffers cycling so that
+// nothing is cache-resident (bench.py --launch-shapes): contiguous runs of 256 KiB per XCD are the
+// best or within 1.5 % of it from 16 MiB to 256 MiB (copy 6.34 against 6.25 TB/s with 16 KiB stripes
+// at 256 MiB); from 1 GiB on, 1 MiB runs are 3-6 % faster than anything below 512 KiB (each XCD's
+// address translations then cover a page at a time instead of every page of the array).
+constexpr long long kStripeBytes = 256 << 10;
+constexpr long long kStripeBytesBigArrays = 1 << 20;
+constexpr unsigned long long kBigArrayBytes = 512ull << 20;
+
+// The tuned stripe (or the one for the array's size class), shrunk for arrays too short to give
+// every XCD at least stripes_per_xcd stripes of it.
+static unsigned long long stripe_for(unsigned long long num_bytes, int num_xcds, const Tuning& t) {
+    unsigned long long stripe = t.stripe_bytes > 0 ? (unsigned long long)t.stripe_bytes
+                              : (unsigned long long)(num_bytes >= kBigArrayBytes ? kStripeBytesBigArrays : kStripeBytes);
+    while (stripe > 4096 && stripe * (unsigned long long)t.stripes_per_xcd * (unsigned)num_xcds > num_bytes) stripe >>= 1;
+    return stripe;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -135,10 +166,15 @@ __global__ void sa_probe_xcd(unsigned char* wg_xcd) {
     }
 }
 
+static int g_num_devices = -1;
+
+// Makes `want` the calling thread's device for a scope.  With a single device there is nothing to
+// switch, and the runtime is not asked.
 struct ScopedDevice {
     int prev = -1;
     bool switched = false;
     explicit ScopedDevice(int want) {
+        if (g_num_devices == 1) return;
         if (hipGetDevice(&prev) == hipSuccess && prev != want) switched = hipSetDevice(want) == hipSuccess;
     }
     ~ScopedDevice() {
@@ -148,7 +184,7 @@ struct ScopedDevice {
 
 struct DeviceContext {
     int device = -1;
-    bool ready = false;
+    std::atomic<bool> ready{false};   // set last in initialize(); read by threads that did not run it
     int num_cus = 0;
     int num_xcds = 1;
     int cus_per_xcd = 0;
@@ -164,13 +200,13 @@ struct DeviceContext {
     void initialize();
 };
 
-static int g_num_devices = -1;
 static std::once_flag g_devices_once;
 static std::vector<std::unique_ptr<DeviceContext>> g_contexts;
 
 static int stripe_hash_mask(int num_xcds) {
     // the address bits that select the owning XCD of a byte: log2(num_xcds) bits above the stripe
-    long long stripe = g_tune.stripe_bytes;
+    const long long tuned = g_tune[0].load(std::memory_order_relaxed);
+    long long stripe = tuned > 0 ? tuned : kStripeBytes;
     long long mask = 0;
     for (long long x = 1; x < num_xcds; x <<= 1) mask |= stripe * x;
     return (int)(mask & 0x7fffffff);
@@ -252,11 +288,12 @@ void DeviceContext::initialize() {
         pool->set_trim_thresholds(total_bytes / 5, total_bytes / 40);
     }
     apply_config(pool.get());
-    ready = true;
+    ready.store(true, std::memory_order_release);
 }
 
-static DeviceContext* get_context(int device = -1) {
-    load_tuning_from_env_once();
+// Counts the devices and makes their (still uninitialised) contexts, once.  After it returns the
+// vector is never resized again, so any thread may walk it.
+static void ensure_contexts() {
     std::call_once(g_devices_once, [] {
         int n = 0;
         if (hipGetDeviceCount(&n) != hipSuccess) {
@@ -269,6 +306,18 @@ static DeviceContext* get_context(int device = -1) {
             g_contexts.back()->device = i;
         }
     });
+}
+
+// Every context some call has initialised so far.
+template <typename F>
+static void for_each_ready_context(F f) {
+    ensure_contexts();
+    for (auto& c : g_contexts) if (c && c->ready.load(std::memory_order_acquire)) f(*c);
+}
+
+static DeviceContext* get_context(int device = -1) {
+    load_tuning_from_env_once();
+    ensure_contexts();
     if (g_num_devices <= 0) {
         set_error("no HIP device is visible");
         return nullptr;
@@ -283,7 +332,7 @@ static DeviceContext* get_context(int device = -1) {
     }
     DeviceContext* ctx = g_contexts[device].get();
     std::call_once(ctx->once, [ctx] { ctx->initialize(); });
-    if (!ctx->ready) {
+    if (!ctx->ready.load(std::memory_order_acquire)) {
         set_error("device %d failed to initialise", device);
         return nullptr;
     }
@@ -295,15 +344,25 @@ static DeviceContext* get_context(int device = -1) {
 // ---------------------------------------------------------------------------------------------
 
 constexpr int kMaxDevices = 16;
-constexpr int kVariants = 8;
+// variant = wide_index | beyond_cache << 1 | in_place << 2 | unaligned << 3
+constexpr int kVariants = 16;
+constexpr int kVariantWide = 1, kVariantBeyond = 2, kVariantInPlace = 4, kVariantUnaligned = 8;
+constexpr int kMaxKernels = 1 << 16;
+constexpr int kMaxSegments = 8;          // SA_MAX_SEGMENTS of the kernel template
 
+// One compiled instantiation.  Filled under its entry's mutex, then published through an atomic
+// pointer and never changed or freed: a launch on any thread may hold it for as long as it likes,
+// and launches already queued on the device keep their module.  A change of a compiled-in knob
+// publishes a new one; the old module stays loaded.
 struct CompiledKernel {
     hipModule_t module = nullptr;
     hipFunction_t fn = nullptr;
+    hipFunction_t fn_batch = nullptr;
     int vgprs = 0, sgprs = 0;
     int occupancy = 0;          // workgroups per CU the hardware can hold
     int tile_vectors = 0;       // from the module's sideaware_kernel_meta
     int owner_is_o0 = 0;
+    int wg_threads = 256;       // the workgroup size it was compiled for
     bool failed = false;
     unsigned generation = 0;
 };
@@ -311,17 +370,19 @@ struct CompiledKernel {
 struct KernelEntry {
     std::string header;         // fixed at registration
     int default_groups = 0;     // fixed at registration; 0: decide from occupancy
-    // Guards function_name and compiled[]: a first-use compile of one op (hundreds of
+    // Serialises the compiles of this op: a first-use compile of one op (hundreds of
     // milliseconds) does not hold up launches of the others.
     std::mutex mu;
-    std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`
-    // [device * kVariants + variant]; variant = wide_index | beyond_cache << 1 | in_place << 2.
-    // Fixed size: launches keep pointers into it while other threads compile other variants.
-    std::array<CompiledKernel, kMaxDevices * kVariants> compiled;
+    std::string function_name = "sideaware_elementwise";   // or the header's `#define KERNEL_NAME x`; under mu
+    std::vector<std::unique_ptr<CompiledKernel>> owned;    // everything ever compiled for this op; under mu
+    std::atomic<CompiledKernel*> ready[kMaxDevices * kVariants];
+    KernelEntry() { for (auto& r : ready) r.store(nullptr, std::memory_order_relaxed); }
 };
 
-static std::mutex g_kernels_mu;
-static std::vector<std::unique_ptr<KernelEntry>> g_kernels;
+// Entries are published once and never removed, so a launch looks its op up without a lock.
+static std::atomic<KernelEntry*> g_entries[kMaxKernels];
+static std::atomic<int> g_entry_count{0};
+static std::mutex g_registry_mu;                          // registration only
 static std::unordered_map<std::string, int> g_header_to_id;
 
 // Finds `#define KERNEL_NAME identifier` in an op header.
@@ -336,148 +397,235 @@ static std::string kernel_name_of(const std::string& header) {
     return end > pos ? header.substr(pos, end - pos) : "sideaware_elementwise";
 }
 
-static void ensure_builtin_locked() {
-    if (!g_kernels.empty()) return;
-    auto e = std::make_unique<KernelEntry>();
-    e->header = kMemcpyHeader;
-    e->function_name = kernel_name_of(e->header);
-    g_kernels.push_back(std::move(e));
+static int publish_entry_locked(const std::string& header, int default_groups) {
+    const int id = g_entry_count.load(std::memory_order_relaxed);
+    if (id >= kMaxKernels) return -1;
+    auto* e = new KernelEntry();        // lives until the process ends
+    e->header = header;
+    e->function_name = kernel_name_of(header);
+    e->default_groups = default_groups > 0 ? default_groups : 0;
+    g_entries[id].store(e, std::memory_order_release);
+    g_entry_count.store(id + 1, std::memory_order_release);
+    return id;
 }
 
-static std::string config_block(int variant, int num_xcds, int num_cus) {
-    load_tuning_from_env_once();
+static void ensure_builtin() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        std::lock_guard<std::mutex> g(g_registry_mu);
+        publish_entry_locked(kMemcpyHeader, 0);           // kernel id 0
+    });
+}
+
+static std::string config_block(int variant, int num_xcds, int num_cus, const Tuning& t) {
     std::string s;
     s += "#define SA_NUM_XCD " + std::to_string(num_xcds) + "\n";
-    s += "#define SA_WG_THREADS " + std::to_string(g_tune.wg_threads) + "\n";
-    s += "#define SA_NT_STORE " + std::to_string(g_tune.nt_store) + "\n";
+    s += "#define SA_WG_THREADS " + std::to_string(t.wg_threads) + "\n";
+    s += "#define SA_NT_STORE " + std::to_string(t.nt_store) + "\n";
+    s += "#define SA_MAX_SEGMENTS " + std::to_string(kMaxSegments) + "\n";
     // Names the reference injects (sideaware.cu:789-794); kept so headers that mention them compile.
     s += "#define MAX_SM " + std::to_string(num_cus) + "\n";
     s += "#define HASH " + std::to_string((stripe_hash_mask(num_xcds) | (1 << 21)) / 16) + "\n";
     s += "#define SA_BEYOND_CACHE " + std::to_string((variant >> 1) & 1) + "\n";
     s += "#define SA_IN_PLACE " + std::to_string((variant >> 2) & 1) + "\n";
-    s += (variant & 1) ? "using size_type = long long;\nconstexpr bool aligned_2MiB = false;\n"
-                       : "using size_type = int;\nconstexpr bool aligned_2MiB = true;\n";
+    // As in the reference (sideaware.cu:792-794, 1386-1388): `aligned_2MiB` is true only in the
+    // instantiation that launches with 2 MiB-aligned i0 and o0 below 2 GiB are routed to.
+    s += (variant & kVariantWide) ? "using size_type = long long;\n" : "using size_type = int;\n";
+    s += (variant & (kVariantWide | kVariantUnaligned)) ? "constexpr bool aligned_2MiB = false;\n"
+                                                        : "constexpr bool aligned_2MiB = true;\n";
     return s;
 }
 
-static std::string full_source(const std::string& header, int variant, int num_xcds, int num_cus) {
-    return config_block(variant, num_xcds, num_cus) + "\n" + header + "\n" + kKernelTemplate;
+static std::string full_source(const std::string& header, int variant, int num_xcds, int num_cus, const Tuning& t) {
+    return config_block(variant, num_xcds, num_cus, t) + "\n" + header + "\n" + kKernelTemplate;
 }
 
-// Returns the compiled function for (id, variant) on ctx's device, building it on first use
-// (sideaware.cu:772-813).  Null after a failed compile; the failure is reported once.
 static KernelEntry* find_entry(int kernel_id) {
-    std::lock_guard<std::mutex> g(g_kernels_mu);
-    ensure_builtin_locked();
-    if (kernel_id < 0 || kernel_id >= (int)g_kernels.size()) {
+    ensure_builtin();
+    if (kernel_id < 0 || kernel_id >= g_entry_count.load(std::memory_order_acquire)) {
         set_error("kernel id %d was never created", kernel_id);
         return nullptr;
     }
-    return g_kernels[kernel_id].get();      // entries are never removed
+    return g_entries[kernel_id].load(std::memory_order_acquire);
 }
 
-static CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant, KernelEntry** entry = nullptr) {
-    KernelEntry* found = find_entry(kernel_id);
-    if (entry) *entry = found;
-    if (!found) return nullptr;
-    KernelEntry& e = *found;
+// Builds the instantiation (sideaware.cu:772-813) and publishes it, successful or not: a failed
+// compile is reported once and remembered.
+static const CompiledKernel* build_kernel(DeviceContext* ctx, int kernel_id, KernelEntry& e, int variant, unsigned gen) {
     std::lock_guard<std::mutex> g(e.mu);
-    if (ctx->device >= kMaxDevices) {
-        set_error("device %d is beyond the %d devices this build keeps kernels for", ctx->device, kMaxDevices);
+    std::atomic<CompiledKernel*>& slot = e.ready[(size_t)ctx->device * kVariants + (size_t)variant];
+    if (CompiledKernel* have = slot.load(std::memory_order_acquire)) {
+        if (have->generation == gen) return have->failed ? nullptr : have;      // another thread was first
+    }
+    e.owned.push_back(std::make_unique<CompiledKernel>());
+    CompiledKernel& k = *e.owned.back();
+    k.generation = gen;
+    const Tuning t = tuning_snapshot();
+    k.wg_threads = (int)t.wg_threads;
+    auto give_up = [&]() -> const CompiledKernel* {
+        k.failed = true;
+        k.fn = k.fn_batch = nullptr;
+        slot.store(&k, std::memory_order_release);
         return nullptr;
-    }
-    CompiledKernel& k = e.compiled[(size_t)ctx->device * kVariants + (size_t)(variant & (kVariants - 1))];
-    unsigned gen = g_tune_generation.load();
-    if (k.generation != gen) {
-        if (k.module) (void)hipModuleUnload(k.module);
-        k = CompiledKernel();
-        k.generation = gen;
-    }
-    if (k.fn) return &k;
-    if (k.failed) return nullptr;
+    };
 
-    CompileResult r = compile_for_gfx950(full_source(e.header, variant, ctx->num_xcds, ctx->num_cus));
+    const std::string source = full_source(e.header, variant, ctx->num_xcds, ctx->num_cus, t);
+    CompileResult r = compile_for_gfx950(source);
     if (!r.log.empty()) std::fprintf(stderr, "sideaware: compiler log for kernel %d:\n%s\n", kernel_id, r.log.c_str());
     if (!r.ok) {
-        k.failed = true;
         set_error("kernel %d (variant %d) failed to compile", kernel_id, variant);
-        return nullptr;
+        return give_up();
     }
+    // What the instantiation says about itself is read from the code object on the host: how many
+    // vectors make a tile, which array's address defines ownership (the launch planner needs
+    // both), and what its entry point is called (the header text may not say: a header that is
+    // only `#include "file"`, example_llmc_rope.cu:138).
+    auto read_self_description = [&](const std::vector<char>& code) {
+        int meta[4] = {0, 0, 0, 0};
+        char name[128] = {0};
+        if (read_code_object_symbol(code, "sideaware_kernel_meta", meta, sizeof meta) != sizeof meta || meta[0] <= 0) return false;
+        const size_t n = read_code_object_symbol(code, "sideaware_kernel_name", name, sizeof name - 1);
+        if (n > 1 && name[0]) e.function_name = name;                 // e.mu is held
+        k.tile_vectors = meta[0];
+        k.owner_is_o0 = meta[2];
+        return true;
+    };
+    // Loading a module is not a stream operation, but a thread that is capturing a stream in the
+    // default (global) mode may not call it: switch this thread to the relaxed mode for the load,
+    // so that an op whose first use falls inside a capture still compiles.
     ScopedDevice guard(ctx->device);
+    hipStreamCaptureMode capture_mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&capture_mode) == hipSuccess;
+    if (!exchanged) (void)hipGetLastError();
     hipError_t err = hipModuleLoadData(&k.module, r.code.data());
     if (err != hipSuccess && r.from_disk_cache) {
         // a cached code object the runtime refuses (damaged file, another driver): build it again
         (void)hipGetLastError();
         k.module = nullptr;
-        r = compile_for_gfx950(full_source(e.header, variant, ctx->num_xcds, ctx->num_cus), "gfx950",
-                               /*use_disk_cache=*/false);
+        r = compile_for_gfx950(source, "gfx950", /*use_disk_cache=*/false);
         err = r.ok ? hipModuleLoadData(&k.module, r.code.data()) : hipErrorInvalidImage;
     }
-    if (err == hipSuccess) {
-        // The module itself says what its entry point is called: the header text may not (a
-        // header that is only `#include "file"`, example_llmc_rope.cu:138).
-        char name[128] = {0};
-        hipDeviceptr_t name_ptr = nullptr;
-        size_t name_bytes = 0;
-        if (hipModuleGetGlobal(&name_ptr, &name_bytes, k.module, "sideaware_kernel_name") == hipSuccess &&
-            name_bytes > 1 && name_bytes < sizeof name &&
-            hipMemcpyDtoH(name, name_ptr, name_bytes) == hipSuccess && name[0]) {
-            e.function_name = name;               // e.mu is held
-        } else {
-            (void)hipGetLastError();
-        }
-        err = hipModuleGetFunction(&k.fn, k.module, e.function_name.c_str());
+    if (err == hipSuccess && !read_self_description(r.code)) {
+        set_error("kernel %d (variant %d): the code object does not describe its tile size", kernel_id, variant);
+        if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&capture_mode);
+        return give_up();
     }
+    if (err == hipSuccess) err = hipModuleGetFunction(&k.fn, k.module, e.function_name.c_str());
+    if (err == hipSuccess) err = hipModuleGetFunction(&k.fn_batch, k.module, (e.function_name + "_batch").c_str());
+    if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&capture_mode);
     if (err != hipSuccess) {
-        k.failed = true;
-        k.fn = nullptr;
         set_error("kernel %d (variant %d) failed to load: %s", kernel_id, variant, hipGetErrorString(err));
         (void)hipGetLastError();
-        return nullptr;
-    }
-    // The instantiation says how many vectors make a tile and which array's address defines
-    // ownership; the launch planner needs both.
-    {
-        hipDeviceptr_t meta_ptr = nullptr;
-        size_t meta_bytes = 0;
-        int meta[4] = {0, 0, 0, 0};
-        err = hipModuleGetGlobal(&meta_ptr, &meta_bytes, k.module, "sideaware_kernel_meta");
-        if (err == hipSuccess && meta_bytes >= sizeof meta) err = hipMemcpyDtoH(meta, meta_ptr, sizeof meta);
-        if (err != hipSuccess || meta[0] <= 0) {
-            k.failed = true;
-            k.fn = nullptr;
-            set_error("kernel %d (variant %d): cannot read its tile size: %s", kernel_id, variant, hipGetErrorString(err));
-            (void)hipGetLastError();
-            return nullptr;
-        }
-        k.tile_vectors = meta[0];
-        k.owner_is_o0 = meta[2];
+        return give_up();
     }
     (void)hipFuncGetAttribute(&k.vgprs, HIP_FUNC_ATTRIBUTE_NUM_REGS, k.fn);
     int occ = 0;
-    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&occ, k.fn, (int)g_tune.wg_threads, 0) != hipSuccess) {
+    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&occ, k.fn, k.wg_threads, 0) != hipSuccess) {
         (void)hipGetLastError();
         occ = 0;
     }
     k.occupancy = occ;
+    slot.store(&k, std::memory_order_release);
     return &k;
 }
 
+// The compiled function for (id, variant) on ctx's device: two atomic loads when it exists.
+// Null after a failed compile.
+static const CompiledKernel* get_kernel(DeviceContext* ctx, int kernel_id, int variant, KernelEntry** entry = nullptr) {
+    KernelEntry* e = find_entry(kernel_id);
+    if (entry) *entry = e;
+    if (!e) return nullptr;
+    if (ctx->device >= kMaxDevices) {
+        set_error("device %d is beyond the %d devices this build keeps kernels for", ctx->device, kMaxDevices);
+        return nullptr;
+    }
+    variant &= kVariants - 1;
+    const unsigned gen = g_tune_generation.load(std::memory_order_acquire);
+    const CompiledKernel* k = e->ready[(size_t)ctx->device * kVariants + (size_t)variant].load(std::memory_order_acquire);
+    if (k && k->generation == gen) return k->failed ? nullptr : k;
+    return build_kernel(ctx, kernel_id, *e, variant, gen);
+}
+
 static int register_header(const char* header, int default_groups) {
-    std::lock_guard<std::mutex> g(g_kernels_mu);
-    ensure_builtin_locked();
+    ensure_builtin();
     if (!header || !*header) return 0;
     std::string text(header);
+    std::lock_guard<std::mutex> g(g_registry_mu);
     auto it = g_header_to_id.find(text);
     if (it != g_header_to_id.end()) return it->second;
-    auto e = std::make_unique<KernelEntry>();
-    e->header = text;
-    e->function_name = kernel_name_of(text);
-    e->default_groups = default_groups > 0 ? default_groups : 0;
-    g_kernels.push_back(std::move(e));
-    int id = (int)g_kernels.size() - 1;
+    const int id = publish_entry_locked(text, default_groups);
+    if (id < 0) {
+        set_error("more than %d kernels were created", kMaxKernels);
+        return 0;
+    }
     g_header_to_id.emplace(std::move(text), id);
     return id;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Launcher
+// ---------------------------------------------------------------------------------------------
+
+// What the device side calls sa_segment_args / sa_batch_args (elementwise_kernel.hip.inc).
+struct SegmentArgs {
+    long long num_vectors;
+    void* out[4];
+    const void* in[4];
+    void* mem;
+    long long full_tiles, b0, u_count, run;
+    int val;
+    unsigned int r;
+    int tail_block;
+    unsigned int first_block;
+};
+struct BatchArgs {
+    SegmentArgs seg[kMaxSegments];
+    unsigned int count;
+    unsigned int blocks_end[kMaxSegments];
+    unsigned int reserved;
+};
+static_assert(sizeof(SegmentArgs) == 128 && sizeof(BatchArgs) == 128 * kMaxSegments + 8 + 4 * kMaxSegments,
+              "the device side declares the same layout");
+
+// The instantiation a launch over these arrays needs.  Index width: 32-bit below 2 GiB, 64-bit from
+// there on.  Cache class: arrays whose result fits the Infinity Cache (written plainly, so the next
+// kernel finds it there) and larger ones (everything streams).  In place (o0 written over i0) is a
+// class of its own below the cache size: see the template's notes on cache policy.  A base that is
+// not 2 MiB-aligned gets the instantiation whose `aligned_2MiB` is false, as in the reference
+// (sideaware.cu:1386-1388), which sends such launches to its 64-bit variant; here the index stays
+// 32 bits wide and only the constant differs.
+static int variant_for(size_t num_bytes, size_t cache_class_bytes, const void* out0, const void* in0, const Tuning& t) {
+    const int wide = num_bytes >= (2ull << 30) ? kVariantWide : 0;
+    const int beyond = cache_class_bytes > (unsigned long long)t.cache_bytes ? kVariantBeyond : 0;
+    const int in_place = (!beyond && out0 != nullptr && out0 == in0) ? kVariantInPlace : 0;
+    constexpr uintptr_t kMask = (2u << 20) - 1;
+    const bool unaligned = (((uintptr_t)out0 | (uintptr_t)in0) & kMask) != 0;
+    return wide | beyond | in_place | ((unaligned && !wide) ? kVariantUnaligned : 0);
+}
+
+// Workgroups per XCD for a persistent launch, or 0 for one workgroup per tile.  The caller's
+// parallel_groups / forced_per_side, or the header's default, fix a persistent grid of
+// (CUs per XCD) x groups; otherwise the tuning decides between one workgroup per tile and a
+// persistent grid sized from the kernel's occupancy.
+static long long slots_wanted_for(const DeviceContext* ctx, const CompiledKernel* k, int default_groups,
+                                  int parallel_groups, int forced_per_side, const Tuning& t) {
+    int per_xcd = ctx->cus_per_xcd;
+    if (forced_per_side > 0 && forced_per_side < per_xcd) per_xcd = forced_per_side;
+    int groups = parallel_groups > 0 ? parallel_groups : default_groups;
+    if (groups <= 0 && forced_per_side <= 0 && t.one_shot) return 0;
+    if (groups <= 0) {
+        groups = k->occupancy > 0 ? k->occupancy : 4;
+        if (groups > t.groups_cap) groups = (int)t.groups_cap;
+    }
+    return (long long)per_xcd * groups;
+}
+
+static bool check_vector_alignment(const char* what, const void* out0, const void* in0, size_t num_bytes) {
+    if ((uintptr_t)out0 % 16 || (uintptr_t)in0 % 16 || num_bytes % 16) {
+        set_error("%s: out0 (%p), in0 (%p) and num_bytes (%zu) must be multiples of 16", what, out0, in0, num_bytes);
+        return false;
+    }
+    return true;
 }
 
 }  // namespace sideaware
@@ -541,9 +689,7 @@ int sideaware_free(void* ptr) {
 
 size_t sideaware_release_unused(void) {
     size_t total = 0;
-    for (auto& c : g_contexts) {
-        if (c && c->ready) total += c->pool->release_unused();
-    }
+    for_each_ready_context([&](DeviceContext& c) { total += c.pool->release_unused(); });
     return total;
 }
 
@@ -553,7 +699,12 @@ int sideaware_create_kernel_advanced(const char* header, bool precompile, int de
     int id = register_header(header, default_num_groups);
     if (precompile) {
         if (DeviceContext* ctx = get_context()) {
-            for (int v = 0; v <= 4; v++) get_kernel(ctx, id, v);     // both index widths x both size classes, and in place
+            // every instantiation a launch can ask for: both index widths, both cache classes, in
+            // place, and bases that are not 2 MiB-aligned
+            static const int kAll[] = {0, kVariantInPlace, kVariantBeyond, kVariantWide | kVariantBeyond,
+                                       kVariantUnaligned, kVariantUnaligned | kVariantInPlace,
+                                       kVariantUnaligned | kVariantBeyond};
+            for (int v : kAll) get_kernel(ctx, id, v);
         }
     }
     return id;
@@ -572,58 +723,26 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     if (num_bytes == 0 || (out0 == nullptr && in0 == nullptr)) return;
     DeviceContext* ctx = get_context(device);
     if (!ctx) return;
-    if ((uintptr_t)out0 % 16 || (uintptr_t)in0 % 16 || num_bytes % 16) {
-        set_error("elementwise: out0 (%p), in0 (%p) and num_bytes (%zu) must be multiples of 16",
-                  out0, in0, num_bytes);
-        return;
-    }
+    if (!check_vector_alignment("elementwise", out0, in0, num_bytes)) return;
 
-    // Lazily compiled instantiations per op.  Index width: 32-bit below 2 GiB, 64-bit from there on (the
-    // reference also sends bases that are not 2 MiB-aligned to its 64-bit variant,
-    // sideaware.cu:1386-1388; here the base only shifts the planner's b0, whatever its alignment).
-    // Cache class: arrays whose result fits the Infinity Cache (written plainly, so the next kernel
-    // finds it there) and larger ones (everything streams).
-    // In place (o0 written over i0) is a class of its own below the cache size: see the template's
-    // notes on cache policy.  Beyond it everything streams already.
-    const int wide = num_bytes >= (2ull << 30) ? 1 : 0;
-    const int beyond = num_bytes > (unsigned long long)g_tune.cache_bytes ? 2 : 0;
-    const int in_place = (!beyond && out0 != nullptr && out0 == in0) ? 4 : 0;
-    const int variant = wide | beyond | in_place;
-
+    const Tuning t = tuning_snapshot();
+    const int variant = variant_for(num_bytes, num_bytes, out0, in0, t);
+    const bool wide = variant & kVariantWide;
     KernelEntry* entry = nullptr;
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant, &entry);
+    const CompiledKernel* k = get_kernel(ctx, kernel_id, variant, &entry);
     if (!k) return;
-    const int default_groups = entry->default_groups;
-    // Workgroups per XCD.  The caller's parallel_groups / forced_per_side, or the header's
-    // default, fix a persistent grid of (CUs per XCD) x groups; otherwise the tuning decides
-    // between one workgroup per tile and a persistent grid sized from the kernel's occupancy.
-    int per_xcd = ctx->cus_per_xcd;
-    if (forced_per_side > 0 && forced_per_side < per_xcd) per_xcd = forced_per_side;
-    int groups = parallel_groups > 0 ? parallel_groups : default_groups;
-    long long slots_wanted;
-    if (groups > 0 || forced_per_side > 0 || !g_tune.one_shot) {
-        if (groups <= 0) {
-            groups = k->occupancy > 0 ? k->occupancy : 4;
-            if (groups > g_tune.groups_cap) groups = (int)g_tune.groups_cap;
-        }
-        slots_wanted = (long long)per_xcd * groups;
-    } else {
-        slots_wanted = 0;
-    }
 
     const long long num_vectors = (long long)(num_bytes / 16);
-    // The ownership stripe: the tuned size, shrunk for arrays too short to give every XCD at least
-    // ~32 stripes of it (one XCD can be a stripe ahead of another).
-    unsigned long long stripe = (unsigned long long)g_tune.stripe_bytes;
-    while (stripe > 4096 && stripe * 32 * ctx->num_xcds > num_bytes) stripe >>= 1;
     const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0);
-    LaunchPlan plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds, stripe,
-                                  g_tune.slot_run, slots_wanted);
-    const unsigned grid = plan.grid;
+    const LaunchPlan plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,
+                                        stripe_for(num_bytes, ctx->num_xcds, t), t.slot_run,
+                                        slots_wanted_for(ctx, k, entry->default_groups, parallel_groups, forced_per_side, t));
 
     long long nv64 = num_vectors, ft64 = plan.full_tiles, b064 = plan.b0, uc64 = plan.u_count, run64 = plan.run;
     int nv32 = (int)num_vectors, ft32 = (int)plan.full_tiles, b032 = (int)plan.b0, uc32 = (int)plan.u_count,
         run32 = (int)plan.run;
+    unsigned int r = plan.r;
+    int tail_block = plan.tail_block;
     int* mem = (int*)sideband_memory;
     void* args[17];
     args[0] = wide ? (void*)&nv64 : (void*)&nv32;
@@ -641,15 +760,93 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     args[12] = wide ? (void*)&b064 : (void*)&b032;
     args[13] = wide ? (void*)&uc64 : (void*)&uc32;
     args[14] = wide ? (void*)&run64 : (void*)&run32;
-    args[15] = &plan.r;
-    args[16] = &plan.tail_block;
+    args[15] = &r;
+    args[16] = &tail_block;
 
     ScopedDevice guard(ctx->device);
-    hipError_t err = hipModuleLaunchKernel(k->fn, grid, 1, 1, (unsigned)g_tune.wg_threads, 1, 1, 0,
+    hipError_t err = hipModuleLaunchKernel(k->fn, plan.grid, 1, 1, (unsigned)k->wg_threads, 1, 1, 0,
                                            (hipStream_t)stream, args, nullptr);
     if (err != hipSuccess) {
         set_error("elementwise: launch of kernel %d failed: %s", kernel_id, hipGetErrorString(err));
         (void)hipGetLastError();
+    }
+}
+
+void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideaware_segment* segments,
+                                 int device, sideaware_stream_t stream) {
+    if (num_segments <= 0 || !segments) return;
+    DeviceContext* ctx = get_context(device);
+    if (!ctx) return;
+    const Tuning t = tuning_snapshot();
+
+    // Segments with nothing to do are dropped, as a single launch of them would be
+    // (sideaware.cu:1366); the rest go out in groups of at most kMaxSegments per launch.
+    for (int first = 0; first < num_segments;) {
+        const sideaware_segment* group[kMaxSegments];
+        int count = 0;
+        size_t total_bytes = 0, largest = 0;
+        bool all_in_place = true, any_unaligned = false;
+        while (first < num_segments && count < kMaxSegments) {
+            const sideaware_segment& g = segments[first++];
+            if (g.num_bytes == 0 || (g.out[0] == nullptr && g.in[0] == nullptr)) continue;
+            if (!check_vector_alignment("elementwise_batch", g.out[0], g.in[0], g.num_bytes)) return;
+            group[count++] = &g;
+            total_bytes += g.num_bytes;
+            largest = g.num_bytes > largest ? g.num_bytes : largest;
+            all_in_place = all_in_place && g.out[0] != nullptr && g.out[0] == g.in[0];
+            any_unaligned = any_unaligned || ((((uintptr_t)g.out[0] | (uintptr_t)g.in[0]) & ((2u << 20) - 1)) != 0);
+        }
+        if (count == 0) continue;
+        // One instantiation serves the whole launch: the widest index any segment needs, the cache
+        // class of everything the launch touches together, in place only if every segment is.
+        int variant = largest >= (2ull << 30) ? kVariantWide : 0;
+        if (total_bytes > (unsigned long long)t.cache_bytes) variant |= kVariantBeyond;
+        else if (all_in_place) variant |= kVariantInPlace;
+        if (any_unaligned && !(variant & kVariantWide)) variant |= kVariantUnaligned;
+
+        KernelEntry* entry = nullptr;
+        const CompiledKernel* k = get_kernel(ctx, kernel_id, variant, &entry);
+        if (!k) return;
+        BatchArgs batch;
+        std::memset(&batch, 0, sizeof batch);
+        batch.count = (unsigned)count;
+        unsigned long long blocks = 0;
+        for (int i = 0; i < count; i++) {
+            const sideaware_segment& g = *group[i];
+            SegmentArgs& a = batch.seg[i];
+            const long long num_vectors = (long long)(g.num_bytes / 16);
+            const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]);
+            const LaunchPlan plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,
+                                                stripe_for(g.num_bytes, ctx->num_xcds, t), t.slot_run,
+                                                slots_wanted_for(ctx, k, entry->default_groups, 0, 0, t));
+            a.num_vectors = num_vectors;
+            for (int j = 0; j < 4; j++) { a.out[j] = g.out[j]; a.in[j] = g.in[j]; }
+            a.mem = g.sideband_memory;
+            a.full_tiles = plan.full_tiles;
+            a.b0 = plan.b0;
+            a.u_count = plan.u_count;
+            a.run = plan.run;
+            a.val = g.sideband_value;
+            a.r = plan.r;
+            a.tail_block = plan.tail_block;
+            a.first_block = (unsigned)blocks;
+            blocks += plan.grid;
+            batch.blocks_end[i] = (unsigned)blocks;
+        }
+        for (int i = count; i < kMaxSegments; i++) batch.blocks_end[i] = (unsigned)blocks;
+        if (blocks == 0 || blocks > 0x7fffffffull) {
+            set_error("elementwise_batch: %llu workgroups do not fit one grid", blocks);
+            return;
+        }
+        void* args[1] = {&batch};
+        ScopedDevice guard(ctx->device);
+        hipError_t err = hipModuleLaunchKernel(k->fn_batch, (unsigned)blocks, 1, 1, (unsigned)k->wg_threads, 1, 1, 0,
+                                               (hipStream_t)stream, args, nullptr);
+        if (err != hipSuccess) {
+            set_error("elementwise_batch: launch of kernel %d failed: %s", kernel_id, hipGetErrorString(err));
+            (void)hipGetLastError();
+            return;
+        }
     }
 }
 
@@ -674,7 +871,7 @@ void sideaware_alloc_threshold(size_t threshold) {
         g_pending_threshold = threshold;
         g_have_pending_threshold = true;
     }
-    for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
+    for_each_ready_context([](DeviceContext& c) { apply_config(c.pool.get()); });
 }
 
 void sideaware_prealloc_config(int extra_required, int extra_alloc) {
@@ -689,7 +886,7 @@ void sideaware_free_mapped_thresholds(size_t start_threshold, size_t end_thresho
         g_pending_trim[1] = end_threshold;
         g_have_pending_trim = true;
     }
-    for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
+    for_each_ready_context([](DeviceContext& c) { apply_config(c.pool.get()); });
 }
 
 void sideaware_reserve_limit(size_t bytes) {
@@ -698,7 +895,7 @@ void sideaware_reserve_limit(size_t bytes) {
         g_pending_limit = bytes;
         g_have_pending_limit = true;
     }
-    for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
+    for_each_ready_context([](DeviceContext& c) { apply_config(c.pool.get()); });
 }
 
 void sideaware_arena_bytes(size_t bytes) {
@@ -707,7 +904,7 @@ void sideaware_arena_bytes(size_t bytes) {
         g_pending_arena = bytes;
         g_have_pending_arena = true;
     }
-    for (auto& c : g_contexts) if (c && c->ready) apply_config(c->pool.get());
+    for_each_ready_context([](DeviceContext& c) { apply_config(c.pool.get()); });
 }
 
 void sideaware_write_sass(const char* filename) { set_isa_dump_file(filename ? filename : ""); }
@@ -767,7 +964,9 @@ void sideaware_clear_error(void) {
 
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity) {
     std::string hdr = header && *header ? header : kMemcpyHeader;
-    CompileResult r = compile_for_gfx950(full_source(hdr, variant & (kVariants - 1), kDefaultXcds, kDefaultCUs));
+    load_tuning_from_env_once();
+    CompileResult r = compile_for_gfx950(full_source(hdr, variant & (kVariants - 1), kDefaultXcds, kDefaultCUs,
+                                                     tuning_snapshot()));
     if (log && log_capacity) {
         std::snprintf(log, log_capacity, "%s", r.log.c_str());
     }
@@ -782,7 +981,8 @@ const char* sideaware_config_block(int variant) {
     static std::string text[kVariants];
     std::lock_guard<std::mutex> g(mu);
     const int v = variant & (kVariants - 1);
-    text[v] = config_block(v, kDefaultXcds, kDefaultCUs);
+    load_tuning_from_env_once();
+    text[v] = config_block(v, kDefaultXcds, kDefaultCUs, tuning_snapshot());
     return text[v].c_str();
 }
 
@@ -790,12 +990,13 @@ int sideaware_kernel_info(int kernel_id, int variant, int* out) {
     DeviceContext* ctx = get_context();
     if (!ctx || !out) return 1;
     KernelEntry* entry = nullptr;
-    CompiledKernel* k = get_kernel(ctx, kernel_id, variant & (kVariants - 1), &entry);
+    const CompiledKernel* k = get_kernel(ctx, kernel_id, variant & (kVariants - 1), &entry);
     if (!k) return 1;
     int groups = entry->default_groups;
     if (groups <= 0) {
         groups = k->occupancy > 0 ? k->occupancy : 4;
-        if (groups > g_tune.groups_cap) groups = (int)g_tune.groups_cap;
+        const long long cap = tuning_snapshot().groups_cap;
+        if (groups > cap) groups = (int)cap;
     }
     out[0] = k->vgprs;
     out[1] = k->sgprs;
@@ -817,13 +1018,15 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity) {
 int sideaware_tune(const char* key, long long value) {
     load_tuning_from_env_once();
     std::lock_guard<std::mutex> g(g_tune_mu);
-    long long* slot = tune_slot(key);
+    std::atomic<long long>* slot = tune_slot(key);
     if (!slot) return 1;
     if (!std::strcmp(key, "wg_threads") && (value < 64 || value > 1024 || (value & (value - 1)))) return 1;
-    if (!std::strcmp(key, "stripe_bytes") && (value < 4096 || value > (1ll << 30) || (value & (value - 1)))) return 1;
+    if (!std::strcmp(key, "stripe_bytes") && value != 0 &&
+        (value < 4096 || value > (1ll << 30) || (value & (value - 1)))) return 1;
     if (!std::strcmp(key, "slot_run") && (value < 0 || value > (1 << 20))) return 1;
-    if (*slot != value) {
-        *slot = value;
+    if (!std::strcmp(key, "stripes_per_xcd") && (value < 1 || value > (1 << 20))) return 1;
+    if (slot->load() != value) {
+        slot->store(value);
         const bool compiled_in = !std::strcmp(key, "nt_store") || !std::strcmp(key, "wg_threads");
         if (compiled_in) g_tune_generation++;      // compiled kernels are rebuilt on their next use
     }
@@ -833,8 +1036,8 @@ int sideaware_tune(const char* key, long long value) {
 long long sideaware_tune_get(const char* key) {
     load_tuning_from_env_once();
     std::lock_guard<std::mutex> g(g_tune_mu);
-    long long* slot = tune_slot(key);
-    return slot ? *slot : -1;
+    std::atomic<long long>* slot = tune_slot(key);
+    return slot ? slot->load() : -1;
 }
 
 }  // extern "C"

@@ -47,7 +47,8 @@ _ROPE_TYPES = {
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
                 layout: str = "qkv", backward: bool = False, unrolled: int | None = 2,
                 reverse_order: bool = False, evict_input: bool = True,
-                stream_input: bool | None = None, stream_output: bool | None = None) -> bytes:
+                stream_input: bool | None = None, stream_output: bool | None = None,
+                heads_at_launch: bool = False) -> bytes:
     """RoPE forward (or backward) in place or out of place.
 
     layout "qkv":   one tensor (B, T, n_q + 2*n_kv, head_dim); q and k heads are rotated, the
@@ -58,6 +59,10 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
 
     in0/out0 is the activation, in1 the fp32 table (T, head_dim/2, 2) of (cos, sin) pairs.
     ``num_bytes`` at launch is the byte size of the activation tensor.
+
+    ``heads_at_launch`` (layout "heads" only): the number of heads per token is not baked into the
+    text but read from the launch's ``sideband_value``, so one compiled kernel serves q and k of a
+    grouped-query model and both can go out in one batched launch (``n_q`` is then ignored).
     """
     if dtype not in _ROPE_TYPES:
         raise ValueError("dtype must be 'fp32', 'bf16' or 'fp16'")
@@ -71,11 +76,14 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     half = head_dim // 2
     if half % pairs_per_vec:
         raise ValueError("head_dim/2 must be a multiple of %d for %s" % (pairs_per_vec, dtype))
+    if heads_at_launch and layout != "heads":
+        raise ValueError("heads_at_launch needs layout 'heads'")
     total_heads = n_q + 2 * n_kv if layout == "qkv" else n_q
     rotated_heads = n_q + n_kv if layout == "qkv" else n_q
     sign_a, sign_b = ("+", "-") if backward else ("-", "+")
 
-    name = "sideaware_rope_%s_%s_%s_t%d_h%d_%d_d%d" % ("bwd" if backward else "fwd", dtype, layout, T, n_q,
+    name = "sideaware_rope_%s_%s_%s_t%d_h%s_%d_d%d" % ("bwd" if backward else "fwd", dtype, layout, T,
+                                                        "N" if heads_at_launch else str(n_q),
                                                         n_kv if layout == "qkv" else 0, head_dim)
     lines = ["#define KERNEL_NAME %s\n" % name, decl]
     if stream_input is not None:
@@ -109,6 +117,24 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
         "}\n" % (widen % "in0.x", widen % "in0.y", sign_a, sign_b, narrow % "y_re", narrow % "y_im"))
     # A 16-byte vector holds pairs_per_vec consecutive pairs of one head of one token, so one
     # decode serves the whole vector: the table row of the token, at the head-local pair.
+    if heads_at_launch:
+        # every head is rotated; the only thing the head count decides is where a token's row ends
+        lines.append(
+            "#define CUSTOM_IDX_FUNC\n"
+            "__device__ __forceinline__ bool indexing(size_type vec_idx, int vec_size,\n"
+            "                         size_type &idx_i0, size_type &idx_i1,\n"
+            "                         size_type &idx_i2, size_type &idx_i3, int* mem, int val) {\n"
+            "    const size_type pair = vec_idx * vec_size;\n"
+            "    const size_type row = (pair / rope_half) / (size_type)val;      // val: heads per token\n"
+            "    const int token = (int)(row % rope_T);\n"
+            "    const int local = (int)(pair % rope_half);\n"
+            "    idx_i0 = vec_idx;\n"
+            "    idx_i1 = (size_type)((token * rope_half + local) / vec_size);\n"
+            "    idx_i2 = 0;\n"
+            "    idx_i3 = 0;\n"
+            "    return false;\n"
+            "}\n")
+        return "".join(lines).encode()
     lines.append(
         "#define CUSTOM_IDX_FUNC\n"
         "__device__ __forceinline__ bool indexing(size_type vec_idx, int vec_size,\n"

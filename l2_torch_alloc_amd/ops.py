@@ -8,6 +8,7 @@ even and sin at odd columns.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Dict, Optional, Tuple
 
@@ -93,6 +94,55 @@ def rope_forward_heads(x, freqs, out=None):
 
 def rope_backward_heads(dout, freqs, out=None):
     return _rope(dout, freqs, out, 0, 0, "heads", True)
+
+
+class _Segment(ctypes.Structure):
+    """``sideaware_segment`` of include/sideaware.h."""
+    _fields_ = [("num_bytes", ctypes.c_size_t), ("out", ctypes.c_void_p * 4), ("inp", ctypes.c_void_p * 4),
+                ("sideband_memory", ctypes.c_void_p), ("sideband_value", ctypes.c_int)]
+
+
+def elementwise_batch(kernel_id: int, segments) -> None:
+    """One launch over several arrays of the same op.  ``segments`` is a sequence of
+    ``(num_bytes, outs, ins, sideband_tensor_or_None, sideband_value)`` with ``outs`` / ``ins``
+    sequences of up to four tensors (or None)."""
+    arr = (_Segment * len(segments))()
+    for seg, (num_bytes, outs, ins, sideband, value) in zip(arr, segments):
+        seg.num_bytes = num_bytes
+        for i, t in enumerate(outs):
+            seg.out[i] = wrapper._check(t, "out%d" % i) or None
+        for i, t in enumerate(ins):
+            seg.inp[i] = wrapper._check(t, "in%d" % i) or None
+        seg.sideband_memory = sideband.data_ptr() if sideband is not None else None
+        seg.sideband_value = int(value)
+    device, stream = torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream
+    wrapper.library().sideaware_elementwise_batch(kernel_id, len(arr), arr, device, stream)
+
+
+def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool):
+    first = tensors[0]
+    assert first.dim() == 4, "activations are (B, T, heads, head_dim)"
+    T, head_dim = first.shape[1], first.shape[3]
+    dtype = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}.get(first.dtype)
+    if dtype is None:
+        raise TypeError("RoPE storage is float32, bfloat16 or float16")
+    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    for t in tensors:
+        assert t.dim() == 4 and t.shape[1] == T and t.shape[3] == head_dim and t.dtype == first.dtype
+    key = ("rope_heads_at_launch", T, head_dim, dtype, backward)
+    kid = _kernel(key, lambda: headers.rope_header(T, 0, 0, head_dim, dtype, "heads", backward, heads_at_launch=True))
+    elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], None, t.shape[2]) for t in tensors])
+    return tensors
+
+
+def rope_forward_heads_many(tensors, freqs):
+    """Rotates several (B, T, heads, head_dim) tensors in place in ONE launch: q and k of a
+    grouped-query model (different head counts, same T, head_dim and dtype) share a grid."""
+    return _rope_heads_many(list(tensors), freqs, False)
+
+
+def rope_backward_heads_many(tensors, freqs):
+    return _rope_heads_many(list(tensors), freqs, True)
 
 
 def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[torch.Tensor] = None):

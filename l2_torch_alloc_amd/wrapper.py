@@ -64,6 +64,7 @@ _SIGNATURES = {
     "sideaware_num_sm_side1": (_ci, []),
     "sideaware_min_sm_per_side": (_ci, []),
     "sideaware_hash_mask": (_ci, []),
+    "sideaware_elementwise_batch": (None, [_ci, _ci, _vp, _ci, _vp]),
     "sideaware_reserve_limit": (None, [_sz]),
     "sideaware_arena_bytes": (None, [_sz]),
     "sideaware_num_xcds": (_ci, []),
@@ -87,7 +88,7 @@ POOL_STAT_FIELDS = (
     "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
     "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
     "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena",
-    "cache_folds",
+    "cache_folds", "refused_frees",
 )
 
 

@@ -1,6 +1,8 @@
 // Appended after the kernel template: runs the whole grid on the CPU, lane by lane, and checks
 // the result.  stdin carries one case per line:
-// "grid num_vectors base_offset_bytes stripe_log2 slot_run".
+// "grid num_vectors base_offset_bytes stripe_log2 slot_run [segments]".  With segments > 1 the
+// array is cut into that many pieces at arbitrary vector boundaries and all of them go through the
+// batched entry point in one grid (only meaningful for ops that do not look at the element index).
 //
 // Every array is a posix_memalign block of exactly the bytes it needs, 2 MiB-aligned and then
 // shifted by base_offset, so a lane that reads or writes past the end trips AddressSanitizer
@@ -15,13 +17,55 @@
 
 #include "../../l2_torch_alloc_amd/csrc/launch_plan.h"
 
-static unsigned g_stripe_log2 = 14, g_slot_run = 1;
+static unsigned g_stripe_log2 = 14, g_slot_run = 1, g_segments = 1;
 
 // `grid` is the caller's wish, as the launcher's parallel_groups would be: a persistent grid of
 // that many workgroups (rounded to whole XCDs), or 0 for one workgroup per tile.  The plan is made
 // by the same function the launcher uses.
 static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3* o3,
                      const vi0* i0, const vi1* i1, const vi2* i2, const vi3* i3, int* mem, int val) {
+    if (g_segments > 1) {
+        sa_batch_args batch;
+        std::memset(&batch, 0, sizeof batch);
+        batch.count = g_segments;
+        unsigned blocks = 0;
+        for (unsigned s = 0; s < g_segments; s++) {
+            // cut points: increasing, rarely on a tile boundary, some pieces empty when nv is small
+            auto cut = [&](unsigned i) -> long long {
+                if (i == 0) return 0;
+                if (i >= g_segments) return (long long)nv;
+                const long long even = (long long)nv * i / g_segments, next = (long long)nv * (i + 1) / g_segments;
+                const long long c = even + (i * 37) % 5;
+                return c > next ? next : c;
+            };
+            const long long lo = cut(s), n = cut(s + 1) - lo;
+            sa_segment_args& a = batch.seg[s];
+            a.output0 = o0 ? o0 + lo : nullptr; a.output1 = o1 ? o1 + lo : nullptr;
+            a.output2 = o2 ? o2 + lo : nullptr; a.output3 = o3 ? o3 + lo : nullptr;
+            a.input0 = i0 ? i0 + lo : nullptr; a.input1 = i1 ? i1 + lo : nullptr;
+            a.input2 = i2 ? i2 + lo : nullptr; a.input3 = i3 ? i3 + lo : nullptr;
+            a.mem = mem; a.val = val; a.num_vectors = n;
+            const unsigned long long seg_base = sideaware_kernel_meta[2] ? (unsigned long long)a.output0
+                                                                          : (unsigned long long)a.input0;
+            sideaware::LaunchPlan p = sideaware::plan_launch(seg_base, n, sideaware_kernel_meta[0], SA_NUM_XCD,
+                                                             1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
+            a.full_tiles = p.full_tiles; a.b0 = p.b0; a.u_count = p.u_count; a.run = p.run;
+            a.r = p.r; a.tail_block = p.tail_block; a.first_block = blocks;
+            blocks += p.grid;
+            batch.blocks_end[s] = blocks;
+        }
+        for (unsigned s = g_segments; s < SA_MAX_SEGMENTS; s++) batch.blocks_end[s] = blocks;
+        gridDim = {blocks, 1, 1};
+        blockDim = {SA_WG_THREADS, 1, 1};
+        for (unsigned b = 0; b < blocks; b++) {
+            for (unsigned t = 0; t < SA_WG_THREADS; t++) {
+                blockIdx = {b, 0, 0};
+                threadIdx = {t, 0, 0};
+                SA_CONCAT(KERNEL_NAME, _batch)(batch);
+            }
+        }
+        return;
+    }
     const unsigned long long base = sideaware_kernel_meta[2] ? (unsigned long long)o0 : (unsigned long long)i0;
     sideaware::LaunchPlan p = sideaware::plan_launch(base, (long long)nv, sideaware_kernel_meta[0], SA_NUM_XCD,
                                                      1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
@@ -143,13 +187,17 @@ int main() {
     long long nv;
     size_t off;
     int cases = 0, failed = 0;
-    while (std::scanf("%u %lld %zu %u %u", &grid, &nv, &off, &g_stripe_log2, &g_slot_run) == 5) {
+    char line[256];
+    while (std::fgets(line, sizeof line, stdin)) {
+        g_segments = 1;
+        if (std::sscanf(line, "%u %lld %zu %u %u %u", &grid, &nv, &off, &g_stripe_log2, &g_slot_run, &g_segments) < 5) continue;
+        if (g_segments < 1 || g_segments > SA_MAX_SEGMENTS) g_segments = 1;
         cases++;
         int bad = run_case(grid, nv, off);
         if (bad) {
             failed++;
-            std::printf("FAIL grid=%u nv=%lld off=%zu stripe_log2=%u run=%u: %d bad elements\n", grid, nv, off,
-                        g_stripe_log2, g_slot_run, bad);
+            std::printf("FAIL grid=%u nv=%lld off=%zu stripe_log2=%u run=%u segments=%u: %d bad elements\n", grid, nv,
+                        off, g_stripe_log2, g_slot_run, g_segments, bad);
         }
     }
     std::printf("cases=%d failed=%d\n", cases, failed);

@@ -15,7 +15,7 @@ from l2_torch_alloc_amd import headers, wrapper
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-# The 27 entry points of the reference's extern "C" block (sideaware.cu:1278-1524).
+# The 26 entry points of the reference's extern "C" block (sideaware.cu:1278-1524).
 REFERENCE_SYMBOLS = [
     "sideaware_malloc_async", "sideaware_free_async", "sideaware_malloc", "sideaware_free",
     "sideaware_release_unused", "sideaware_malloc_auto", "sideaware_free_auto",
@@ -185,6 +185,55 @@ def test_header_may_include_a_file_relative_to_the_working_directory(lib, tmp_pa
     assert rc != 0 and "error" in log
     rc, log = compile_ok(lib, b'#include "no_such_file.h"\n', 0)
     assert rc != 0 and "no_such_file.h" in log
+
+
+@pytest.mark.parametrize("spelling", [b'#include <my_op.h>\n', b'#  include   "my_op.h"\n', b'#\tinclude<my_op.h>\n'])
+def test_every_spelling_of_a_user_include_bypasses_the_disk_cache(lib, tmp_path, monkeypatch, spelling):
+    # the content of a user's file is not in the cache key, whatever the include looks like
+    monkeypatch.setenv("SIDEAWARE_CACHE_DIR", str(tmp_path / "cache"))
+    (tmp_path / "my_op.h").write_bytes(headers.scale_bias_bf16_header())
+    monkeypatch.chdir(tmp_path)
+    rc, log = compile_ok(lib, spelling, 0)
+    assert rc == 0, log
+    (tmp_path / "my_op.h").write_bytes(b"typedef int o0; this is not C++")
+    rc, log = compile_ok(lib, spelling, 0)
+    assert rc != 0 and "error" in log
+    assert not os.path.isdir(tmp_path / "cache") or os.listdir(tmp_path / "cache") == []
+
+
+def test_headers_of_the_toolchain_are_cached(lib, tmp_path, monkeypatch):
+    monkeypatch.setenv("SIDEAWARE_CACHE_DIR", str(tmp_path / "cache"))
+    rc, log = compile_ok(lib, b"#include <hip/hip_fp16.h>\n#include <cuda_bf16.h>\n" + headers.fill_header(), 0)
+    assert rc == 0, log
+    assert len(os.listdir(tmp_path / "cache")) == 1
+
+
+def test_headers_that_define_the_references_optional_macros_compile(lib):
+    # sideaware.cu:60-79: DISCARD_INPUTS with input_discard[4], DYNAMIC_INDEX_FOR_CONCURRENT_KERNELS,
+    # FORCE_WRONG_SIDE / FORCE_RANDOM_SIDE: accepted, with no effect on gfx950
+    text = lib.sideaware_memcpy_header().decode().replace("#define KERNEL_NAME sideaware_copy", "")
+    header = ("#define DISCARD_INPUTS\nconstexpr bool input_discard[4] = {true, false, false, false};\n"
+              "#define DYNAMIC_INDEX_FOR_CONCURRENT_KERNELS\n#define FORCE_WRONG_SIDE false\n"
+              "#define FORCE_RANDOM_SIDE false\n" + text).encode()
+    for variant in (0, 3, 8):
+        rc, log = compile_ok(lib, header, variant)
+        assert rc == 0, log
+
+
+def test_aligned_2mib_is_true_only_in_the_aligned_32_bit_instantiations(lib):
+    # sideaware.cu:792-794: `aligned_2MiB` goes with the 32-bit index type; a launch whose bases are
+    # not 2 MiB-aligned runs an instantiation in which it is false (variant bit 3)
+    for variant in range(16):
+        block = lib.sideaware_config_block(variant).decode()
+        wide, unaligned = variant & 1, variant & 8
+        assert ("using size_type = long long;" in block) == bool(wide)
+        assert ("constexpr bool aligned_2MiB = true;" in block) == (not wide and not unaligned), variant
+        assert ("constexpr bool aligned_2MiB = false;" in block) == bool(wide or unaligned), variant
+    header = (b"static_assert(!aligned_2MiB, \"this instantiation is for bases that are not 2 MiB-aligned\");\n"
+              + headers.fill_header())
+    assert compile_ok(lib, header, 0)[0] != 0
+    assert compile_ok(lib, header, 8)[0] == 0
+    assert compile_ok(lib, header, 1)[0] == 0
 
 
 REFERENCE_DIR = "/root/reference"

@@ -133,11 +133,17 @@ def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, reverse):
     cases = cases_for(variant, unrolled, rng)
     if case == "MIXED":
         cases = [(g, n, off - off % 64, s, r) for (g, n, off, s, r) in cases]   # halved offsets stay 16 B-aligned
-    text = "".join("%d %d %d %d %d\n" % c for c in cases)
-    proc = subprocess.run([exe], input=text, capture_output=True, text=True, timeout=600,
+        lines = ["%d %d %d %d %d\n" % c for c in cases]
+    else:
+        # every case through the single-array entry point, and a fifth of them again cut into 2..8
+        # segments that share one grid of the batched entry point
+        lines = ["%d %d %d %d %d\n" % c for c in cases]
+        lines += ["%d %d %d %d %d %d\n" % ((min(c[0], 56),) + c[1:] + (rng.choice([2, 3, 5, 8]),))
+                  for c in rng.sample(cases, len(cases) // 5)]
+    proc = subprocess.run([exe], input="".join(lines), capture_output=True, text=True, timeout=600,
                           env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
-    assert "cases=%d failed=0" % len(cases) in proc.stdout
+    assert "cases=%d failed=0" % len(lines) in proc.stdout
 
 
 ROPE_SHAPES = [

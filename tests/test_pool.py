@@ -27,7 +27,7 @@ FIELDS = ("large_hits", "large_misses", "small_hits", "small_carves", "slabs_acq
           "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
           "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
           "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena",
-          "cache_folds")
+          "cache_folds", "refused_frees")
 
 
 def build_harness():
@@ -502,6 +502,39 @@ def test_double_free_and_interior_pointer_are_refused(pool):
     q = pool.alloc(2048)
     assert pool.free(q + 512) != 0                    # not a block start
     assert pool.L.ph_owns(pool.h, q)
+
+
+@pytest.mark.parametrize("arena", [0, 4 * GiB])
+def test_stale_pointers_into_the_pools_own_arenas_never_reach_the_runtime(ph, arena):
+    # A second free of a large region, the base of an arena whose first region was freed, an interior
+    # pointer of a live region and a pointer into free pages are all addresses the runtime's own
+    # free must never see: its free of an arena's base would take the arena away from under the
+    # blocks carved from it.  They are refused and counted; nothing is forwarded.
+    pool = P(ph, capacity=64 * GiB, arena=arena)
+    try:
+        a = pool.alloc(64 * MiB)
+        b = pool.alloc(32 * MiB)
+        assert pool.free(a) == 0
+        pool.clear_log()
+        assert pool.free(a) != 0                      # double free (with arenas: a is the arena's base)
+        assert pool.free(b + 2 * MiB) != 0            # interior pointer of a live region
+        assert pool.free(a + 4 * MiB) != 0            # inside a cached region
+        if arena:
+            assert pool.free(b + 512 * MiB) != 0      # free pages of the arena, never handed out
+        assert not any(l.startswith("foreign") for l in pool.log()), pool.log()
+        st = pool.stats()
+        assert st["foreign_frees"] == 0 and st["refused_frees"] == (4 if arena else 3)
+        # the pool is intact: the cached region comes back, the live one is still live
+        assert pool.alloc(64 * MiB) == a
+        assert pool.L.ph_owns(pool.h, b)
+        # after the cache went back to the driver the old address is foreign again, as it should be
+        assert pool.free(a) == 0 and pool.free(b) == 0
+        pool.L.ph_release_unused(pool.h)
+        pool.clear_log()
+        assert pool.free(a) == 0
+        assert pool.log() == ["foreign %d" % a]
+    finally:
+        pool.close()
 
 
 def test_free_null_and_foreign(pool):
