@@ -291,6 +291,27 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
         run("stripe sweep: library sideaware_memcpy stripe_bytes=%d" % stripe, 2 * nbytes,
             lambda d, s: lib.sideaware_memcpy(d, s, nbytes, 0, stream))
     assert lib.sideaware_tune(b"stripe_bytes", 0) == 0
+    # time against size, per stripe: a straight-line fit separates the steady rate from the cost of
+    # starting and draining a launch
+    if only and any("size fit" in o for o in only):
+        big_src = torch.empty(4 * GiB, dtype=torch.uint8, device="cuda")
+        big_src.view(torch.int64).random_()
+        big_dst = torch.empty(4 * GiB, dtype=torch.uint8, device="cuda")
+        for r in (0, 2, 5, 6, 7, 8, 9):
+            for mib in (64, 128, 256, 512, 1024, 2048):
+                size, slots = mib * MiB, (4 * GiB) // (mib * MiB)
+
+                def cycle():
+                    for j in range(slots):
+                        rc = ceil.hbm_ceiling_tile(big_dst.data_ptr() + j * size, big_src.data_ptr() + j * size, size,
+                                                   1, 256, r, hints["nt"], sink.data_ptr(), stream)
+                        assert rc == 0
+
+                sec = time_region(cycle, max(2, steps // 2), 1) / slots
+                name = "size fit: copy k=1 block=256 stripe=%dKiB nt size=%dMiB" % (4 << r, mib)
+                out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(2 * size, sec), 1)}
+                log("%-58s %9.1f us %8.1f GB/s" % (name, sec * 1e6, gbps(2 * size, sec)))
+        del big_src, big_dst
     # chip-wide phases: one iteration of the whole grid moves grid*block*k*16 bytes each way; the
     # period is swept around the time that takes at 6.2-7.2 TB/s
     for k, block, grid in ((16, 1024, 256), (8, 1024, 512), (8, 1024, 256)):
@@ -394,4 +415,66 @@ def launch_shapes(steps, only=None):
                 out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(total, sec), 1)}
                 log("%-60s %9.2f us %8.1f GB/s" % (name, sec * 1e6, gbps(total, sec)))
     assert lib.sideaware_tune(b"stripe_bytes", 0) == 0 and lib.sideaware_tune(b"stripes_per_xcd", 8) == 0
+    return out
+
+
+# ------------------------------------------------------------------------------------- producer -> consumer, per XCD
+
+def chain_xcd(reps=4, only=None):
+    """Producer -> consumer on the same buffer, meant to be run under `rocprofv3 --pmc` with the per-XCD
+    TCC_HIT / TCC_MISS counters of profiles/xcd_counters.yaml: a copy writes `mid` (stores plain or
+    nontemporal), and at once a second copy reads `mid`, walking each XCD's tiles in the same order
+    or in reverse (`reverse_order`, the reference's knob for exactly this: sideaware.cu:40), so that
+    it starts with what the producer wrote last.  Buffer sets cycle, so nothing but the producer's
+    result can be cache-resident.  Kernel names carry size, store policy and order; per-launch times
+    come from HIP events."""
+    import torch
+    from l2_torch_alloc_amd import headers, wrapper
+    lib, stream = _abi()
+    base = headers.memcpy_header().decode()
+    out = {}
+
+    def kernel(tag, stream_out, reverse, stream_in=1):
+        text = "#define INPUT0_STREAMING %d\n#define OUTPUT_STREAMING %d\n" % (stream_in, stream_out) + base
+        text = text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME " + tag)
+        text = text.replace("constexpr bool reverse_order = false;", "constexpr bool reverse_order = %s;" % ("true" if reverse else "false"))
+        return wrapper.sideaware_create_kernel(text.encode())
+
+    for mib in (8, 32, 64, 128, 256, 512):
+        nbytes = mib * MiB
+        sets = min(24, max(3, (1536 * MiB) // (3 * nbytes)))
+        srcs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(sets)]
+        mids = [torch.empty_like(t) for t in srcs]
+        outs = [torch.empty_like(t) for t in srcs]
+        # the consumer's loads carry the streaming hint, except in the "plainloads" cases
+        cases = [(policy, order, 1) for policy in ("plain", "nt") for order in ("same", "reversed")]
+        cases += [("plain", "same", 0), ("plain", "reversed", 0)]
+        for policy, order, consumer_stream_in in cases:
+                stream_out, reverse = int(policy == "nt"), order == "reversed"
+                name = "%dMiB_%s_%s%s" % (mib, policy, order, "" if consumer_stream_in else "_plainloads")
+                if only and not any(o in name for o in only):
+                    continue
+                producer = kernel("chainP_%s_" % name, stream_out, False)
+                consumer = kernel("chainC_%s_" % name, 1, reverse, consumer_stream_in)
+                evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(sets)]
+                tp = tc = 0.0
+                for rep in range(reps + 1):
+                    for i in range(sets):
+                        e = evs[i]
+                        e[0].record()
+                        lib.sideaware_one_to_one(producer, nbytes, mids[i].data_ptr(), srcs[i].data_ptr(), 0, stream)
+                        e[1].record()
+                        lib.sideaware_one_to_one(consumer, nbytes, outs[i].data_ptr(), mids[i].data_ptr(), 0, stream)
+                        e[2].record()
+                    torch.cuda.synchronize()
+                    if rep:
+                        tp += sum(e[0].elapsed_time(e[1]) for e in evs)
+                        tc += sum(e[1].elapsed_time(e[2]) for e in evs)
+                n = reps * sets
+                ok = all(bool(torch.equal(o, s)) for o, s in zip(outs, srcs))
+                out[name] = {"producer_us": round(tp / n * 1e3, 2), "consumer_us": round(tc / n * 1e3, 2),
+                             "consumer_GBps": round(gbps(2 * nbytes, tc / n * 1e-3), 1), "sets": sets, "bit_exact": ok}
+                log("%-28s producer %8.2f us  consumer %8.2f us (%7.1f GB/s)  %s" % (
+                    name, tp / n * 1e3, tc / n * 1e3, gbps(2 * nbytes, tc / n * 1e-3), "ok" if ok else "WRONG"))
+        del srcs, mids, outs
     return out

@@ -26,7 +26,7 @@ def test_algorithmic_byte_counts():
     assert 2 * (q + k) + table == 673185792
     # measured traffic constants stay within 1 % of those algorithmic bytes
     assert abs(bench.COPY_256MIB_TRAFFIC_BYTES / (2 * 256 * 2 ** 20) - 1) < 0.01
-    assert abs((bench.ROPE_Q_TRAFFIC_BYTES + bench.ROPE_K_TRAFFIC_BYTES) / 673185792 - 1) < 0.01
+    assert abs(bench.ROPE_STEP_TRAFFIC_BYTES / 673185792 - 1) < 0.01
     sizes = bench.churn_sizes()
     assert len(sizes) == 10000 and min(sizes) >= 4096 and max(sizes) <= 512 * 2 ** 20 and all(s % 16 == 0 for s in sizes)
     assert sizes == bench.churn_sizes()                          # seeded
@@ -50,6 +50,11 @@ def test_quick_run_prints_one_json_line_with_roofline_and_cpu_baseline():
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9 and 0.3 < roof["frac"] < 1.0
     assert abs(r["value"] - 2 * 256 * 2 ** 20 / (r["ms_per_step"] * 1e-3) / 1e9) < 1.0
+    rope = r["roofline_rope_bf16"]
+    assert rope["bound"] == "hbm" and rope["peak"] == 8000.0 and 0.3 < rope["frac"] < 1.0
+    assert abs(rope["frac"] - rope["achieved"] / rope["peak"]) < 1e-9
+    assert abs(rope["achieved"] - 673185792 / (rope["ms_per_step"] * 1e-3) / 1e9) < 1.0
+    assert "cycle over 8 distinct" in r["config"]["workload"]
     cpu = r["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] == 1 and cpu["value"] > 0
     assert r["library_error"] is None
