@@ -130,7 +130,8 @@ void sideaware_arena_bytes(size_t bytes);
 int sideaware_num_xcds(void);
 /* 1 when the start-up probe found workgroup i of a launch on XCD i % num_xcds. */
 int sideaware_xcd_dealing_verified(void);
-/* Text of the most recent failure on any thread ("" if none). */
+/* Text of the most recent failure on any thread ("" if none).  The pointer is the calling thread's
+ * own copy, valid until that thread calls again. */
 const char* sideaware_last_error(void);
 void sideaware_clear_error(void);
 /* Compiles header + template for gfx950 without touching a device. variant bit 0: 0 = 32-bit indices
@@ -143,7 +144,8 @@ int sideaware_compile_check(const char* header, int variant, char* log, size_t l
 /* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */
 const char* sideaware_kernel_source(void);
 const char* sideaware_memcpy_header(void);
-/* The configuration block the host would prepend for `variant` with the current tuning. */
+/* The configuration block the host would prepend for `variant` with the current tuning (the
+ * calling thread's own copy, valid until that thread calls again). */
 const char* sideaware_config_block(int variant);
 /* out[0..3] = { VGPRs, SGPRs, workgroups per CU by occupancy, default workgroups per CU }
  * of a compiled kernel; compiles it if needed.  Returns 0 on success. */

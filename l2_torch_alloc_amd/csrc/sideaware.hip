@@ -58,7 +58,6 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
 
 static std::mutex g_err_mu;
 static std::string g_last_error;
-static std::string g_last_error_snapshot;
 
 static void set_error(const char* fmt, ...) {
     char buf[2048];
@@ -952,9 +951,11 @@ int sideaware_num_xcds(void) { DeviceContext* c = get_context(); return c ? c->n
 int sideaware_xcd_dealing_verified(void) { DeviceContext* c = get_context(); return c && c->dealing_verified ? 1 : 0; }
 
 const char* sideaware_last_error(void) {
+    // a copy in the calling thread's own buffer: valid until that thread asks again
+    static thread_local std::string snapshot;
     std::lock_guard<std::mutex> g(g_err_mu);
-    g_last_error_snapshot = g_last_error;
-    return g_last_error_snapshot.c_str();
+    snapshot = g_last_error;
+    return snapshot.c_str();
 }
 
 void sideaware_clear_error(void) {
@@ -977,13 +978,11 @@ const char* sideaware_kernel_source(void) { return kKernelTemplate; }
 const char* sideaware_memcpy_header(void) { return kMemcpyHeader; }
 
 const char* sideaware_config_block(int variant) {
-    static std::mutex mu;
-    static std::string text[kVariants];
-    std::lock_guard<std::mutex> g(mu);
-    const int v = variant & (kVariants - 1);
+    // the text lives in the calling thread's own buffer until that thread asks again
+    static thread_local std::string text;
     load_tuning_from_env_once();
-    text[v] = config_block(v, kDefaultXcds, kDefaultCUs, tuning_snapshot());
-    return text[v].c_str();
+    text = config_block(variant & (kVariants - 1), kDefaultXcds, kDefaultCUs, tuning_snapshot());
+    return text.c_str();
 }
 
 int sideaware_kernel_info(int kernel_id, int variant, int* out) {

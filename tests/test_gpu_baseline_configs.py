@@ -379,3 +379,32 @@ def test_free_of_a_foreign_pointer_is_forwarded_to_the_runtime_in_stream_order(s
     torch.cuda.synchronize()
     assert torch.cuda.mem_get_info()[0] >= free0
     assert sa.sideaware_alloc_stats()["foreign_frees"] == before["foreign_frees"] + 2
+
+
+# --------------------------------------------------------------------------------------- producer -> consumer
+
+@pytest.mark.parametrize("n", [4096 + 24, 12 * MiB + 8, 160 * MiB], ids=["8KiB", "24MiB", "320MiB"])
+def test_producer_then_reversed_consumer_on_the_same_buffer_vs_oracle(sa, n):
+    # the reference's ping-pong (sideaware.cu:40, test.py:211-212): a kernel writes a buffer and the next one reads
+    # it walking each XCD's tiles from the end.  Producer: bf16 y = 1.5 x + 0.25; consumer, reverse_order = true:
+    # z = -0.5 y + 2, in place on y.  Both against the oracle, bit for bit.
+    from l2_torch_alloc_amd import headers, ops
+    lib = sa.library()
+    stream = torch.cuda.current_stream().cuda_stream
+    reversed_text = headers.scale_bias_bf16_header().decode() \
+        .replace("constexpr bool reverse_order = false;", "constexpr bool reverse_order = true;") \
+        .replace("#define KERNEL_NAME sideaware_scale_bias_bf16", "#define KERNEL_NAME test_scale_bias_bf16_reversed")
+    assert "reverse_order = true" in reversed_text
+    consumer = sa.sideaware_create_kernel(reversed_text.encode())
+    x_h = torch.randn(n, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16)
+    x = x_h.cuda()
+    y = torch.empty_like(x)
+    sb1 = torch.tensor([1.5, 0.25], dtype=torch.float32, device="cuda")
+    sb2 = torch.tensor([-0.5, 2.0], dtype=torch.float32, device="cuda")
+    ops.scale_bias_bf16(x, sb1, out=y)
+    lib.sideaware_elementwise(consumer, n * 2, y.data_ptr(), 0, 0, 0, y.data_ptr(), 0, 0, 0, sb2.data_ptr(), 0, 0, 0, 0, stream)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    want = O.scale_bias_bf16(O.scale_bias_bf16(bits(x_h), 1.5, 0.25), -0.5, 2.0)
+    assert np.array_equal(bits(y).reshape(-1), np.asarray(want).reshape(-1))
+    assert np.array_equal(bits(x), bits(x_h))                       # the producer's input is untouched
