@@ -124,6 +124,12 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
 /* Upper bound on the device bytes the pool may hold (0 = none): a request that would pass it is
  * answered like one the device refused (caches are given back, then null). */
 void sideaware_reserve_limit(size_t bytes);
+/* What sideaware_malloc_auto does when nothing can be allocated.  0 (default): return null, the
+ * reference's contract (sideaware.cu:1250-1251).  1: raise a C++ std::runtime_error instead, for
+ * C++ hosts that do not check the pointer: PyTorch's pluggable-allocator shim is one (a null there
+ * becomes a tensor whose data pointer is 0), and the exception reaches Python as a RuntimeError.
+ * Only sideaware_malloc_auto is affected; the entry points that return an error code keep doing so. */
+void sideaware_oom_raises(int enable);
 /* Size of the arenas that large regions are carved from (default 4 GiB); 0 gives every large
  * region a driver allocation of its own, as in the reference. */
 void sideaware_arena_bytes(size_t bytes);

@@ -89,12 +89,7 @@ void Pool::note_reserved(int64_t delta) {
 // Adds a free extent, merging it with free neighbours of the same arena.
 void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
     ExtentIndex& ix = free_[kind];
-    auto erase_size = [&](size_t bytes, uintptr_t a) {
-        auto range = ix.by_size.equal_range(bytes);
-        for (auto it = range.first; it != range.second; ++it) {
-            if (it->second == a) { ix.by_size.erase(it); return; }
-        }
-    };
+    auto erase_size = [&](size_t bytes, uintptr_t a) { ix.by_size.erase({bytes, a}); };
     auto next = ix.by_addr.lower_bound(addr);
     if (next != ix.by_addr.end() && next->second.arena == e.arena && addr + e.bytes == next->first) {
         e.freed_on.merge(next->second.freed_on);
@@ -119,7 +114,7 @@ void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
 // Takes `bytes` from the front of the best-fitting free extent; the remainder stays free.
 bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken) {
     ExtentIndex& ix = free_[kind];
-    auto sit = ix.by_size.lower_bound(bytes);
+    auto sit = ix.by_size.lower_bound({bytes, 0});
     if (sit == ix.by_size.end()) return false;
     *addr = sit->second;
     auto ait = ix.by_addr.find(*addr);
@@ -226,10 +221,7 @@ size_t Pool::release_free_arenas_locked(int kind, size_t down_to, bool device_id
             st_.device_syncs++;
             synced = true;
         }
-        auto range = ix.by_size.equal_range(a->bytes);
-        for (auto sit = range.first; sit != range.second; ++sit) {
-            if (sit->second == (uintptr_t)a->base) { ix.by_size.erase(sit); break; }
-        }
+        ix.by_size.erase({a->bytes, (uintptr_t)a->base});
         ix.by_addr.erase(fit);
         backing_->release(a->base, a->bytes);
         st_.backing_releases++;
@@ -251,18 +243,40 @@ size_t Pool::trim_large_locked(size_t down_to) {
 void* Pool::allocate_large_locked(size_t bytes, void* stream) {
     const size_t rounded = round_large(bytes);
 
+    bool trimmed = false;
     // 1) exact-size reuse, newest first (sideaware.cu:1199-1219)
     auto it = large_cache_.find(rounded);
     if (it == large_cache_.end() || it->second.empty()) {
-        // 2) best fit from the arenas' free extents: no waste, no driver call
-        if (void* p = carve_locked(rounded, stream)) {
-            st_.large_carves++;
-            return p;
+        if (arena_bytes_ != 0) {
+            // 2) with arenas: every cached region goes back into its arena's free extents, where
+            //    neighbours merge, and the request is carved, best fit, from what is free then.  No
+            //    waste, no driver call; a fold costs microseconds.  Folding before every carve (and
+            //    not only when nothing else fits) is what keeps the arenas whole: a cached region
+            //    is a hole its neighbours cannot merge across, and carving around such holes left
+            //    16 GB of a 89 GB pool free yet too fragmented for a 512 MiB request in a churn of
+            //    10,000 requests; folding first, the same churn peaks at 76 GB.
+            //    When cached + free bytes have outgrown their budget the same moment is the
+            //    reference's threshold trim (sideaware.cu:1242): wholly free arenas go home too.
+            if (st_.bytes_cached_large + st_.bytes_free_arena > trim_start_) {
+                trim_large_locked(trim_end_);
+                st_.trims++;
+                trimmed = true;
+            } else if (!large_cache_.empty()) {
+                flush_cache_locked();
+                st_.cache_folds++;
+            }
+            if (void* p = carve_locked(rounded, stream)) {
+                st_.large_carves++;
+                return p;
+            }
+            it = large_cache_.end();
+        } else {
+            // 2') without arenas every region is a backing allocation of its own: the smallest
+            //     cached region at most one eighth larger is handed out whole
+            it = large_cache_.lower_bound(rounded);
+            while (it != large_cache_.end() && it->second.empty()) ++it;
+            if (it != large_cache_.end() && it->first > rounded + rounded / 8) it = large_cache_.end();
         }
-        // 3) the smallest cached region at most one eighth larger, handed out whole
-        it = large_cache_.lower_bound(rounded);
-        while (it != large_cache_.end() && it->second.empty()) ++it;
-        if (it != large_cache_.end() && it->first > rounded + rounded / 8) it = large_cache_.end();
     }
     if (it != large_cache_.end() && !it->second.empty()) {
         LargeBlock blk = it->second.back();
@@ -284,22 +298,10 @@ void* Pool::allocate_large_locked(size_t bytes, void* stream) {
     // 4) a miss.  If cached + free bytes have outgrown their budget, fold the cache into the
     //    arenas and give wholly free arenas back (the reference's threshold trim,
     //    sideaware.cu:1242); what stays free may now fit the request.
-    if (st_.bytes_cached_large + st_.bytes_free_arena > trim_start_) {
+    if (!trimmed && st_.bytes_cached_large + st_.bytes_free_arena > trim_start_) {
         trim_large_locked(trim_end_);
         st_.trims++;
         if (void* p = carve_locked(rounded, stream)) return p;
-    } else if (arena_bytes_ != 0 && !large_cache_.empty()) {
-        // Under the budget, with arenas: cached regions of other sizes are folded back into their
-        // arenas, where neighbours merge, before the driver is asked for more.  A fold costs
-        // microseconds, a driver allocation a thousand times that, and the pool then holds about
-        // what is live instead of every size it has ever seen.
-        flush_cache_locked();
-        st_.cache_folds++;
-        if (void* p = carve_locked(rounded, stream)) {
-            st_.large_misses--;
-            st_.large_carves++;
-            return p;
-        }
     }
     if (new_arena_locked(kLargeArenas, rounded)) return carve_locked(rounded, stream);
 

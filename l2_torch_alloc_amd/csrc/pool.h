@@ -11,14 +11,17 @@
 // caching behaviour:
 //
 //   large  (size >= threshold): a 2 MiB-aligned region, size rounded up to 2 MiB.  Freed regions
-//          go to an exact-size LIFO reuse cache, as in the reference.  A size that is not cached
-//          is carved, best fit, from the free extents of multi-GiB arenas (a driver allocation
-//          costs hundreds of microseconds; a carve costs one), or served by a cached region at
-//          most 1/8 larger, handed out whole, or, failing that, from the arenas again after the
-//          whole cache was folded back into them.  When cached plus free bytes outgrow the
-//          thresholds the cache is folded back into the arenas and wholly free arenas return to
-//          the backing store; the reference's four-step out-of-memory ladder ends in null
-//          (sideaware.cu:1233-1252);
+//          go to an exact-size LIFO reuse cache, as in the reference: the same size comes back at
+//          the same address.  A size that is not cached first folds the whole cache back into the
+//          free extents of the multi-GiB arenas the regions were carved from (neighbours merge),
+//          and is then carved, best fit and lowest address first, from what is free: no driver
+//          call (a driver allocation costs hundreds of microseconds, a fold and a carve one or
+//          two), and no holes that a cached neighbour keeps from merging.  Only when no free run
+//          is long enough is the driver asked, for a new arena.  When cached plus free bytes
+//          outgrow the thresholds, wholly free arenas return to the backing store; the
+//          reference's four-step out-of-memory ladder ends in null (sideaware.cu:1233-1252).
+//          Without arenas (arena size 0: every region a backing allocation of its own, the
+//          reference's shape) a cached region at most 1/8 larger is handed out whole instead;
 //   small  (size <  threshold): 512 B-granular size classes carved from slabs, so the common
 //          small request never reaches the driver (the reference forwards these to
 //          cudaMallocAsync, sideaware.cu:1326-1339).  Slabs are themselves carved from arenas
@@ -35,6 +38,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <set>
 #include <unordered_map>
 #include <vector>
 
@@ -173,9 +177,10 @@ private:
         Arena* arena = nullptr;    // null: a backing allocation of its own
         std::vector<uint8_t> in_use;   // one flag per block: catches double frees
     };
-    struct ExtentIndex {           // the free extents of one kind of arena, by address and by size
+    struct ExtentIndex {           // the free extents of one kind of arena, by address and by (size, address)
         std::map<uintptr_t, Extent> by_addr;
-        std::multimap<size_t, uintptr_t> by_size;
+        std::set<std::pair<size_t, uintptr_t>> by_size;   // best fit = first entry not below (bytes, 0): among
+                                                           // the smallest extents that fit, the lowest address
     };
     enum { kLargeArenas = 0, kSlabArenas = 1 };
     struct FreeSmall {

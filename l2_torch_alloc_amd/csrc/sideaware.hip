@@ -6,11 +6,13 @@
 #include <atomic>
 #include <cctype>
 #include <cstdarg>
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -55,6 +57,10 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
 // ---------------------------------------------------------------------------------------------
 // Errors: recorded, printed, never thrown
 // ---------------------------------------------------------------------------------------------
+
+// What sideaware_malloc_auto does when the pool has nothing left: return null (the reference's
+// contract, sideaware.cu:1250-1251) or raise a C++ exception (for a host that does not check).
+static std::atomic<int> g_oom_raises{0};
 
 static std::mutex g_err_mu;
 static std::string g_last_error;
@@ -641,8 +647,18 @@ extern "C" {
 
 void* sideaware_malloc_auto(size_t size, int device, sideaware_stream_t stream) {
     DeviceContext* ctx = get_context(device);
-    if (!ctx) return nullptr;
-    return ctx->pool->allocate(size, stream, /*always_large=*/false);
+    void* p = ctx ? ctx->pool->allocate(size, stream, /*always_large=*/false) : nullptr;
+    if (!p && size != 0 && g_oom_raises.load(std::memory_order_relaxed)) {
+        // PyTorch's pluggable-allocator shim does not look at the pointer it gets: a null would
+        // become a tensor whose data pointer is 0, and the first kernel on it a GPU fault.  Its
+        // frames are C++, so an exception thrown here arrives in Python as a RuntimeError.
+        char msg[256];
+        std::snprintf(msg, sizeof msg, "sideaware: out of memory: tried to allocate %zu bytes on device %d "
+                      "(see sideaware_alloc_stats)", size, device);
+        set_error("%s", msg);
+        throw std::runtime_error(msg);
+    }
+    return p;
 }
 
 void sideaware_free_auto(void* ptr, size_t size, int device, sideaware_stream_t stream) {
@@ -737,34 +753,36 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
                                         stripe_for(num_bytes, ctx->num_xcds, t), t.slot_run,
                                         slots_wanted_for(ctx, k, entry->default_groups, parallel_groups, forced_per_side, t));
 
-    long long nv64 = num_vectors, ft64 = plan.full_tiles, b064 = plan.b0, uc64 = plan.u_count, run64 = plan.run;
-    int nv32 = (int)num_vectors, ft32 = (int)plan.full_tiles, b032 = (int)plan.b0, uc32 = (int)plan.u_count,
-        run32 = (int)plan.run;
-    unsigned int r = plan.r;
-    int tail_block = plan.tail_block;
-    int* mem = (int*)sideband_memory;
-    void* args[17];
-    args[0] = wide ? (void*)&nv64 : (void*)&nv32;
-    args[1] = &out0;
-    args[2] = &out1;
-    args[3] = &out2;
-    args[4] = &out3;
-    args[5] = &in0;
-    args[6] = &in1;
-    args[7] = &in2;
-    args[8] = &in3;
-    args[9] = &mem;
-    args[10] = &sideband_value;
-    args[11] = wide ? (void*)&ft64 : (void*)&ft32;
-    args[12] = wide ? (void*)&b064 : (void*)&b032;
-    args[13] = wide ? (void*)&uc64 : (void*)&uc32;
-    args[14] = wide ? (void*)&run64 : (void*)&run32;
-    args[15] = &r;
-    args[16] = &tail_block;
+    // The kernel's arguments, laid out as the device code declares them (natural alignment, in
+    // order) and handed to the runtime as one block.
+    struct Args32 { int nv; void* p[9]; int val; int ft, b0, uc, run; unsigned int r; int tail; };
+    struct Args64 { long long nv; void* p[9]; int val; long long ft, b0, uc, run; unsigned int r; int tail; };
+    static_assert(offsetof(Args32, tail) == 104 && offsetof(Args64, tail) == 124, "kernel argument layout");
+    union { Args32 a32; Args64 a64; } args;
+    size_t args_bytes;
+    void* const ptrs[9] = {out0, out1, out2, out3, (void*)in0, (void*)in1, (void*)in2, (void*)in3, sideband_memory};
+    if (wide) {
+        Args64& a = args.a64;
+        a.nv = num_vectors;
+        std::memcpy(a.p, ptrs, sizeof ptrs);
+        a.val = sideband_value;
+        a.ft = plan.full_tiles; a.b0 = plan.b0; a.uc = plan.u_count; a.run = plan.run;
+        a.r = plan.r; a.tail = plan.tail_block;
+        args_bytes = offsetof(Args64, tail) + sizeof(int);
+    } else {
+        Args32& a = args.a32;
+        a.nv = (int)num_vectors;
+        std::memcpy(a.p, ptrs, sizeof ptrs);
+        a.val = sideband_value;
+        a.ft = (int)plan.full_tiles; a.b0 = (int)plan.b0; a.uc = (int)plan.u_count; a.run = (int)plan.run;
+        a.r = plan.r; a.tail = plan.tail_block;
+        args_bytes = offsetof(Args32, tail) + sizeof(int);
+    }
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &args_bytes, HIP_LAUNCH_PARAM_END};
 
     ScopedDevice guard(ctx->device);
     hipError_t err = hipModuleLaunchKernel(k->fn, plan.grid, 1, 1, (unsigned)k->wg_threads, 1, 1, 0,
-                                           (hipStream_t)stream, args, nullptr);
+                                           (hipStream_t)stream, nullptr, extra);
     if (err != hipSuccess) {
         set_error("elementwise: launch of kernel %d failed: %s", kernel_id, hipGetErrorString(err));
         (void)hipGetLastError();
@@ -896,6 +914,8 @@ void sideaware_reserve_limit(size_t bytes) {
     }
     for_each_ready_context([](DeviceContext& c) { apply_config(c.pool.get()); });
 }
+
+void sideaware_oom_raises(int enable) { g_oom_raises.store(enable ? 1 : 0, std::memory_order_relaxed); }
 
 void sideaware_arena_bytes(size_t bytes) {
     {

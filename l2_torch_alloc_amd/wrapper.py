@@ -66,6 +66,7 @@ _SIGNATURES = {
     "sideaware_hash_mask": (_ci, []),
     "sideaware_elementwise_batch": (None, [_ci, _ci, _vp, _ci, _vp]),
     "sideaware_reserve_limit": (None, [_sz]),
+    "sideaware_oom_raises": (None, [_ci]),
     "sideaware_arena_bytes": (None, [_sz]),
     "sideaware_num_xcds": (_ci, []),
     "sideaware_xcd_dealing_verified": (_ci, []),
@@ -176,6 +177,9 @@ def sideaware_init(path: str = DEFAULT_LIBRARY, install_allocator: bool = True) 
         _allocator_installed = True
     if _lib is None:
         _lib = bind(path)
+    # PyTorch does not check the pointer its pluggable allocator returns: have an exhausted pool
+    # raise (a RuntimeError in Python) instead of handing PyTorch a null
+    _lib.sideaware_oom_raises(1)
     _register_ops()
     _refresh_metadata()
     # the reference prints this line when initialisation is done (example_wrapper.py:109); here it

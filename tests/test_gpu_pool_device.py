@@ -77,19 +77,27 @@ def test_release_unused_gives_memory_back(sa):
             + after["bytes_cached_small"]) <= after["bytes_reserved"]
 
 
-def test_out_of_memory_is_a_null_pointer_not_a_crash(sa):
+def test_out_of_memory_is_a_null_pointer_for_c_callers_and_an_exception_for_pytorch(sa):
     # More than the device holds: every step of the ladder fails and the entry point returns null
     # (sideaware.cu:1250-1251 ends the same way).  PyTorch's pluggable-allocator shim does not check
-    # the pointer, so the tensor it builds has a null data pointer; it is never touched here.
+    # the pointer and would build a tensor with a null data pointer, so for PyTorch (sideaware_init
+    # switches this on) the entry point raises instead, and torch.empty fails loudly.
     total = torch.cuda.get_device_properties(0).total_memory
     lib = sa.library()
     before = sa.sideaware_alloc_stats()["failures"]
-    p = lib.sideaware_malloc_auto(total + (8 << 30), 0, None)
-    assert p is None
-    assert sa.sideaware_alloc_stats()["failures"] == before + 1
-    t = torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
-    assert t.data_ptr() == 0
-    del t
+    lib.sideaware_oom_raises(0)                  # the reference's contract; a C caller (ctypes is one) gets null
+    try:
+        p = lib.sideaware_malloc_auto(total + (8 << 30), 0, None)
+        assert p is None
+        assert sa.sideaware_alloc_stats()["failures"] == before + 1
+        t = torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
+        assert t.data_ptr() == 0                 # what PyTorch makes of a null: never touched here
+        del t
+    finally:
+        lib.sideaware_oom_raises(1)
+    with pytest.raises(RuntimeError, match="sideaware: out of memory"):
+        torch.empty(total + (8 << 30), dtype=torch.uint8, device="cuda")
+    assert "out of memory" in sa.sideaware_last_error()
     out = ctypes.c_void_p(1)
     assert lib.sideaware_malloc(ctypes.byref(out), total + (8 << 30)) == 2      # hipErrorOutOfMemory
     assert out.value is None
@@ -104,6 +112,7 @@ def test_reserve_limit_acts_like_a_full_device(sa):
     lib.sideaware_release_unused()
     st = sa.sideaware_alloc_stats()
     lib.sideaware_reserve_limit(st["bytes_reserved"] + 256 * MiB)
+    lib.sideaware_oom_raises(0)                  # ctypes calls below: null, not a C++ exception
     try:
         ok = lib.sideaware_malloc_auto(128 * MiB, 0, None)            # free arena space, or a small new arena
         assert ok and ok % (2 * MiB) == 0
@@ -113,6 +122,7 @@ def test_reserve_limit_acts_like_a_full_device(sa):
         lib.sideaware_free_auto(ok, 128 * MiB, 0, None)
     finally:
         lib.sideaware_reserve_limit(0)
+        lib.sideaware_oom_raises(1)
         lib.sideaware_clear_error()
     z = torch.empty(512 * MiB, dtype=torch.uint8, device="cuda")
     assert z.data_ptr() % (2 * MiB) == 0

@@ -286,12 +286,21 @@ def test_regions_are_carved_from_one_arena_and_coalesce(ph):
         # the first request needed the driver (a miss); the next two were carved from what it brought
         assert st["large_misses"] == 1 and st["large_carves"] == 2
         assert st["arenas_acquired"] == 1 and st["bytes_free_arena"] == 16 * MiB
-        # a size that is not cached is carved from the arena's free tail, not from the driver
+        # a freed region comes back exactly while it is cached (LIFO, as in the reference) ...
+        pool.free(b)
+        assert pool.stats()["bytes_cached_large"] == 16 * MiB
+        assert pool.alloc(16 * MiB) == b and pool.stats()["large_hits"] == 1
+        # ... and a request of a size that is not cached folds the cache back into the arena first and
+        # is carved, best fit, from what is free then: here from the hole b leaves, not from the
+        # 16 MiB tail, and not from the driver
         pool.free(b)
         d = pool.alloc(10 * MiB)
-        assert d == c + 16 * MiB and pool.stats()["backing_acquires"] == 1
-        # the freed 16 MiB comes back exactly (LIFO cache), not through a carve
-        assert pool.alloc(16 * MiB) == b and pool.stats()["large_hits"] == 1
+        st = pool.stats()
+        assert d == b and st["backing_acquires"] == 1 and st["cache_folds"] == 1 and st["bytes_cached_large"] == 0
+        assert st["bytes_free_arena"] == 6 * MiB + 16 * MiB
+        e = pool.alloc(16 * MiB)
+        assert e == c + 16 * MiB
+        b = e
         # everything freed and folded back: the extents merge into the whole arena, which goes home
         for p in (a, b, c, d):
             pool.free(p)
