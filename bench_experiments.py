@@ -389,6 +389,26 @@ def launch_shapes(steps, only=None):
                 name = "rope bf16 q+k x %d sets tile=%dKiB stripe_bytes=%d" % (sets, 4 * unrolled, stripe)
                 out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(total, sec), 1)}
                 log("%-60s %9.2f us %8.1f GB/s" % (name, sec * 1e6, gbps(total, sec)))
+        # larger workgroups (a compiled-in knob: every kernel is built afresh for it), 4 KiB per workgroup instruction
+        # becomes 8 or 16 KiB
+        for wg in (512, 1024):
+            assert lib.sideaware_tune(b"wg_threads", wg) == 0 and lib.sideaware_tune(b"stripe_bytes", 0) == 0
+            for unrolled in (1, 2):
+                if wg * unrolled * 16 > 16384:
+                    continue
+                kid_q = wrapper.sideaware_create_kernel(headers.rope_header(T, 32, 0, HS, "bf16", "heads", unrolled=unrolled))
+                kid_k = wrapper.sideaware_create_kernel(headers.rope_header(T, 8, 0, HS, "bf16", "heads", unrolled=unrolled))
+
+                def cycle_wg():
+                    for q, k in zip(qs, ks):
+                        lib.sideaware_elementwise(kid_q, q_bytes, q.data_ptr(), 0, 0, 0, q.data_ptr(), fp, 0, 0, 0, 0, 0, 0, 0, stream)
+                        lib.sideaware_elementwise(kid_k, k_bytes, k.data_ptr(), 0, 0, 0, k.data_ptr(), fp, 0, 0, 0, 0, 0, 0, 0, stream)
+
+                sec = time_region(cycle_wg, steps, 2) / sets
+                name = "rope bf16 q+k x %d sets workgroup=%d threads tile=%dKiB stripe by size" % (sets, wg, wg * unrolled * 16 // 1024)
+                out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(total, sec), 1)}
+                log("%-60s %9.2f us %8.1f GB/s" % (name, sec * 1e6, gbps(total, sec)))
+        assert lib.sideaware_tune(b"wg_threads", 256) == 0
         # q and k in one launch (one kernel, the head count travels in the sideband value)
         for unrolled in (1, 2):
             kid = wrapper.sideaware_create_kernel(headers.rope_header(T, 0, 0, HS, "bf16", "heads", unrolled=unrolled,

@@ -137,19 +137,23 @@ static std::atomic<long long>* tune_slot(const char* key) {
 }
 
 // The ownership stripe for an array of num_bytes.  Measured on MI355X with buffers cycling so that
-// nothing is cache-resident (bench.py --launch-shapes): contiguous runs of 256 KiB per XCD are the
-// best or within 1.5 % of it from 16 MiB to 256 MiB (copy 6.34 against 6.25 TB/s with 16 KiB stripes
-// at 256 MiB); from 1 GiB on, 1 MiB runs are 3-6 % faster than anything below 512 KiB (each XCD's
-// address translations then cover a page at a time instead of every page of the array).
-constexpr long long kStripeBytes = 256 << 10;
+// nothing is cache-resident (bench.py --launch-shapes, two runs that agree to 0.5 %): contiguous
+// runs of 128 KiB per XCD are the best from 64 MiB to 256 MiB (copy 6.37 against 6.25 TB/s with 16 KiB
+// stripes at 256 MiB; bf16 RoPE 6.60 against 6.44); at 16 MiB, 256 KiB runs are (4.76 against 4.38);
+// from 1 GiB on, 1 MiB runs are 3-6 % faster than anything below 512 KiB (each XCD's address
+// translations then cover a page at a time instead of every page of the array).
+constexpr long long kStripeBytesSmallArrays = 256 << 10;
+constexpr long long kStripeBytes = 128 << 10;
 constexpr long long kStripeBytesBigArrays = 1 << 20;
+constexpr unsigned long long kSmallArrayBytes = 32ull << 20;
 constexpr unsigned long long kBigArrayBytes = 512ull << 20;
 
 // The tuned stripe (or the one for the array's size class), shrunk for arrays too short to give
 // every XCD at least stripes_per_xcd stripes of it.
 static unsigned long long stripe_for(unsigned long long num_bytes, int num_xcds, const Tuning& t) {
     unsigned long long stripe = t.stripe_bytes > 0 ? (unsigned long long)t.stripe_bytes
-                              : (unsigned long long)(num_bytes >= kBigArrayBytes ? kStripeBytesBigArrays : kStripeBytes);
+                              : (unsigned long long)(num_bytes >= kBigArrayBytes ? kStripeBytesBigArrays
+                                                     : num_bytes >= kSmallArrayBytes ? kStripeBytes : kStripeBytesSmallArrays);
     while (stripe > 4096 && stripe * (unsigned long long)t.stripes_per_xcd * (unsigned)num_xcds > num_bytes) stripe >>= 1;
     return stripe;
 }
