@@ -181,7 +181,7 @@ def ceiling_library():
         raise FileNotFoundError("%s is not built; run `python -m l2_torch_alloc_amd.build`" % path)
     lib = ctypes.CDLL(path)
     vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
-    lib.hbm_ceiling_tile.argtypes = [vp, vp, sz, ci, ci, ci, ci, vp, vp]
+    lib.hbm_ceiling_tile.argtypes = [vp, vp, sz, ci, ci, ci, ci, vp, vp, vp]
     lib.hbm_ceiling_tile.restype = ci
     lib.hbm_ceiling_persistent.argtypes = [vp, vp, sz, ci, ci, ci, ci, ctypes.c_uint, vp, vp]
     lib.hbm_ceiling_persistent.restype = ci
@@ -221,7 +221,7 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
     def tile(k, block, r, flags, read=True, write=True, in_place=False):
         def launch(d, s):
             return ceil.hbm_ceiling_tile(s if in_place else (d if write else None), s if read else None,
-                                         nbytes, k, block, r, flags, sink.data_ptr(), stream)
+                                         nbytes, k, block, r, flags, sink.data_ptr(), None, stream)
         return launch
 
     def persistent(k, block, grid, flags, period, read=True, write=True):
@@ -304,7 +304,7 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
                 def cycle():
                     for j in range(slots):
                         rc = ceil.hbm_ceiling_tile(big_dst.data_ptr() + j * size, big_src.data_ptr() + j * size, size,
-                                                   1, 256, r, hints["nt"], sink.data_ptr(), stream)
+                                                   1, 256, r, hints["nt"], sink.data_ptr(), None, stream)
                         assert rc == 0
 
                 sec = time_region(cycle, max(2, steps // 2), 1) / slots
@@ -312,6 +312,74 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
                 out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(2 * size, sec), 1)}
                 log("%-58s %9.1f us %8.1f GB/s" % (name, sec * 1e6, gbps(2 * size, sec)))
         del big_src, big_dst
+    # the same launches spread over two streams: a launch may start while the one before it drains
+    if only and any("two streams" in o for o in only):
+        n = 256 * MiB
+        k_pairs = 8
+        s_srcs = [torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda") for _ in range(k_pairs)]
+        s_dsts = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(k_pairs)]
+        side = [torch.cuda.Stream(), torch.cuda.Stream()]
+        for st in side:                               # streams are made on first use: not inside a timed region
+            st.wait_stream(torch.cuda.current_stream())
+            torch.cuda.current_stream().wait_stream(st)
+        torch.cuda.synchronize()
+        for label, streams in (("one stream", [torch.cuda.current_stream()]), ("two streams", side)):
+            for i in range(k_pairs):                  # untimed: every stream and buffer has been used once
+                lib.sideaware_memcpy(s_dsts[i].data_ptr(), s_srcs[i].data_ptr(), n, 0, streams[i % len(streams)].cuda_stream)
+            torch.cuda.synchronize()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 6
+            ev0.record()
+            for st in side:
+                st.wait_event(ev0)
+            for rep in range(reps):
+                for i in range(k_pairs):
+                    st = streams[i % len(streams)]
+                    lib.sideaware_memcpy(s_dsts[i].data_ptr(), s_srcs[i].data_ptr(), n, 0, st.cuda_stream)
+            for st in side:
+                torch.cuda.current_stream().wait_stream(st)
+            ev1.record()
+            torch.cuda.synchronize()
+            sec = ev0.elapsed_time(ev1) * 1e-3 / (reps * k_pairs)
+            name = "two streams: library copy 256MiB x 8 pairs, launches on %s" % label
+            out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(2 * n, sec), 1)}
+            log("%-58s %9.1f us %8.1f GB/s" % (name, sec * 1e6, gbps(2 * n, sec)))
+        assert all(bool(torch.equal(d, t)) for d, t in zip(s_dsts, s_srcs))
+        del s_srcs, s_dsts
+    # when does each XCD start and finish its share of a launch?  (device clock, 10 ns ticks; every
+    # workgroup writes its own start and end time, the host reduces them per XCD: workgroup i runs on XCD i % 8)
+    if only and any("xcd spread" in o for o in only):
+        for size_mib, r in ((256, 5), (256, 8), (1024, 8), (64, 5)):
+            size = size_mib * MiB
+            tiles = size // 4096
+            stamps = torch.zeros(2 * tiles, dtype=torch.int64, device="cuda")
+            finish, start, durs, ramp = [], [], [], []
+            for rep in range(10):
+                i = rep % pairs
+                torch.cuda.synchronize()
+                rc = ceil.hbm_ceiling_tile(dsts[i].data_ptr(), srcs[i].data_ptr(), size, 1, 256, r, hints["nt"],
+                                           sink.data_ptr(), stamps.data_ptr(), stream)
+                assert rc == 0
+                torch.cuda.synchronize()
+                t = stamps.view(tiles, 2)
+                t0 = torch.stack([t[x::8, 0].min() for x in range(8)]).cpu().numpy()
+                t1 = torch.stack([t[x::8, 1].max() for x in range(8)]).cpu().numpy()
+                first_done = int(t[:, 1].min())
+                if rep >= 2:
+                    log("   rep %d pair %d: per-XCD finish, us before the last one: %s" % (
+                        rep, i, " ".join("%5.2f" % ((int(t1.max()) - int(v)) / 100.0) for v in t1)))
+                    finish.append((int(t1.max()) - int(t1.min())) / 100.0)
+                    start.append((int(t0.max()) - int(t0.min())) / 100.0)
+                    durs.append((int(t1.max()) - int(t0.min())) / 100.0)
+                    ramp.append((first_done - int(t0.min())) / 100.0)
+            name = "xcd spread: copy %dMiB stripe=%dKiB nt" % (size_mib, 4 << r)
+            out[name] = {"first_start_to_last_end_us": round(sum(durs) / len(durs), 2),
+                         "last_minus_first_xcd_to_finish_us": round(sum(finish) / len(finish), 2),
+                         "worst_us": round(max(finish), 2),
+                         "last_minus_first_xcd_to_start_us": round(sum(start) / len(start), 2),
+                         "first_workgroup_done_after_us": round(sum(ramp) / len(ramp), 2)}
+            log(name, out[name])
+            del stamps
     # chip-wide phases: one iteration of the whole grid moves grid*block*k*16 bytes each way; the
     # period is swept around the time that takes at 6.2-7.2 TB/s
     for k, block, grid in ((16, 1024, 256), (8, 1024, 512), (8, 1024, 256)):

@@ -43,8 +43,13 @@ __device__ __forceinline__ long long striped_tile(unsigned b, unsigned r) {
 
 // One workgroup per tile of K * blockDim.x vectors.  dst == nullptr: read only; src == nullptr:
 // write only; both: copy (dst == src: read-modify-write in place).
+// `stamps` (optional): two device words per workgroup, into which it writes the device clock at
+// its start and at its end (after its stores were acknowledged), so the host can see when each
+// XCD started and finished its share of a launch.
 template <int K, bool NTL, bool NTS, bool CONTIG>
-__global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, unsigned r, int flags, int* sink) {
+__global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, unsigned r, int flags, int* sink,
+                                                    unsigned long long* stamps) {
+    if (stamps && threadIdx.x == 0) stamps[2 * (size_t)blockIdx.x] = wall_clock64();
     const unsigned B = blockDim.x, tid = threadIdx.x;
     const long long tile = striped_tile(blockIdx.x, r);
     const long long base = tile * (long long)(B * K);
@@ -77,6 +82,10 @@ __global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, un
         #pragma unroll
         for (int k = 1; k < K; k++) acc ^= v[k];
         sink_if_magic(acc, sink);
+    }
+    if (stamps && threadIdx.x == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // this wave's stores are acknowledged
+        stamps[2 * (size_t)blockIdx.x + 1] = wall_clock64();
     }
 }
 
@@ -121,7 +130,7 @@ __global__ __launch_bounds__(1024) void persistent_kernel(v4i* dst, const v4i* s
     }
 }
 
-typedef void (*tile_fn)(v4i*, const v4i*, unsigned, int, int*);
+typedef void (*tile_fn)(v4i*, const v4i*, unsigned, int, int*, unsigned long long*);
 typedef void (*persistent_fn)(v4i*, const v4i*, long long, int, unsigned, int*);
 
 template <int K>
@@ -158,9 +167,10 @@ extern "C" {
 const char* hbm_ceiling_last_error(void) { return g_error; }
 
 // One workgroup per tile.  `bytes` must be a multiple of 8 * (k * block * 16) << stripe_log2.
+// `stamps`: null, or two device words per tile that receive each workgroup's start and end time.
 // Returns 0 when the kernel was launched.
 int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block, int stripe_log2, int flags,
-                     int* sink, hipStream_t stream) {
+                     int* sink, unsigned long long* stamps, hipStream_t stream) {
     if (block < 64 || block > 1024 || (block & (block - 1))) return fail("block must be a power of two in 64..1024");
     if (stripe_log2 < 0 || stripe_log2 > 12) return fail("stripe_log2 must be in 0..12");
     if (!dst && !src) return fail("nothing to do");
@@ -180,7 +190,7 @@ int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block,
         default: return fail("k must be 1, 2, 4, 8 or 16");
     }
     hipLaunchKernelGGL(fn, dim3((unsigned)tiles), dim3(block), 0, stream, (v4i*)dst, (const v4i*)src,
-                       (unsigned)stripe_log2, flags, sink);
+                       (unsigned)stripe_log2, flags, sink, stamps);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
 }
