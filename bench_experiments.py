@@ -183,6 +183,8 @@ def ceiling_library():
     vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     lib.hbm_ceiling_tile.argtypes = [vp, vp, sz, ci, ci, ci, ci, vp, vp, vp]
     lib.hbm_ceiling_tile.restype = ci
+    lib.hbm_ceiling_balanced_copy.argtypes = [vp, vp, sz, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), vp, vp]
+    lib.hbm_ceiling_balanced_copy.restype = ci
     lib.hbm_ceiling_persistent.argtypes = [vp, vp, sz, ci, ci, ci, ci, ctypes.c_uint, vp, vp]
     lib.hbm_ceiling_persistent.restype = ci
     lib.hbm_ceiling_last_error.restype = ctypes.c_char_p
@@ -312,6 +314,67 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
                 out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(2 * size, sec), 1)}
                 log("%-58s %9.1f us %8.1f GB/s" % (name, sec * 1e6, gbps(2 * size, sec)))
         del big_src, big_dst
+    # unequal shares per XCD: measure how far ahead of the last XCD each one finishes, give the slow
+    # ones fewer tiles and the fast ones more, and time the copy again
+    if only and any("xcd shares" in o for o in only):
+        import numpy as np
+        for size_mib, r in ((256, 5), (1024, 8)):
+            size = size_mib * MiB
+            own = size // 4096 // 8
+            ci8 = ctypes.c_int * 8
+            equal_cut, zero = ci8(*([own] * 8)), ci8(*([0] * 8))
+
+            def measure_leads(cut, extra, reps=10):
+                slots = own + max(extra)
+                stamps = torch.zeros(2 * 8 * slots, dtype=torch.int64, device="cuda")
+                leads, spans = [], []
+                for rep in range(reps):
+                    i = rep % pairs
+                    stamps.zero_()
+                    torch.cuda.synchronize()
+                    rc = ceil.hbm_ceiling_balanced_copy(dsts[i].data_ptr(), srcs[i].data_ptr(), size, r, cut, extra,
+                                                        stamps.data_ptr(), stream)
+                    assert rc == 0, ceil.hbm_ceiling_last_error()
+                    torch.cuda.synchronize()
+                    assert bool(torch.equal(dsts[i][:size], srcs[i][:size]))
+                    t = stamps.view(8 * slots, 2)
+                    ran = t[:, 1] != 0
+                    ends = np.array([int(t[x::8, 1].max()) for x in range(8)], dtype=np.int64)
+                    start = int(t[:, 0][ran].min())
+                    if rep >= 2:
+                        leads.append((ends.max() - ends) / 100.0)
+                        spans.append((ends.max() - start) / 100.0)
+                return np.mean(leads, axis=0), float(np.mean(spans))
+
+            def timed(cut, extra):
+                def cycle():
+                    for i in range(pairs):
+                        rc = ceil.hbm_ceiling_balanced_copy(dsts[i].data_ptr(), srcs[i].data_ptr(), size, r, cut, extra,
+                                                            None, stream)
+                        assert rc == 0
+                return time_region(cycle, max(steps, 6), 2) / pairs
+
+            leads, span = measure_leads(equal_cut, zero)
+            speed = own / (span - leads)                     # tiles per us of each XCD
+            want = np.floor(speed / speed.sum() * own * 8 + 0.5).astype(int)
+            want[int(np.argmax(want))] += own * 8 - int(want.sum())
+            cut = ci8(*[int(min(own, w)) for w in want])
+            extra = ci8(*[int(max(0, w - own)) for w in want])
+            leads2, span2 = measure_leads(cut, extra)
+            t_equal = [timed(equal_cut, zero), None, None]
+            t_shares = [timed(cut, extra), None, None]
+            for j in (1, 2):
+                t_equal[j] = timed(equal_cut, zero)
+                t_shares[j] = timed(cut, extra)
+            name = "xcd shares: copy %dMiB stripe=%dKiB nt" % (size_mib, 4 << r)
+            out[name] = {"equal_shares_us": [round(x * 1e6, 2) for x in t_equal],
+                         "measured_shares_us": [round(x * 1e6, 2) for x in t_shares],
+                         "equal_GBps": round(gbps(2 * size, min(t_equal)), 1),
+                         "measured_shares_GBps": round(gbps(2 * size, min(t_shares)), 1),
+                         "tiles_per_xcd": [int(w) for w in want], "own": own,
+                         "leads_us_equal": [round(float(x), 2) for x in leads], "span_us_equal": round(span, 2),
+                         "leads_us_shares": [round(float(x), 2) for x in leads2], "span_us_shares": round(span2, 2)}
+            log(name, out[name])
     # the same launches spread over two streams: a launch may start while the one before it drains
     if only and any("two streams" in o for o in only):
         n = 256 * MiB

@@ -89,6 +89,45 @@ __global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, un
     }
 }
 
+// The one-workgroup-per-4-KiB nt copy with unequal shares per XCD.  Workgroups are dealt to the
+// XCDs in turn, so each XCD gets the same number of workgroup slots (own + the largest extra);
+// XCD x does only the first cut[x] of its own tiles, and the tiles the donors leave over are done
+// by the helper slots (slot >= own) of the XCDs with extra[x] > 0, in donor order.
+struct xcd_shares {
+    int cut[8];
+    int extra[8];
+};
+__global__ __launch_bounds__(256) void balanced_copy_kernel(v4i* dst, const v4i* src, unsigned r, int own, xcd_shares sh,
+                                                            unsigned long long* stamps) {
+    const unsigned tid = threadIdx.x, xcd = blockIdx.x & 7u;
+    int slot = (int)(blockIdx.x >> 3);
+    if (stamps && tid == 0) stamps[2 * (size_t)blockIdx.x] = wall_clock64();
+    unsigned owner = xcd;
+    if (slot >= own) {
+        int h = slot - own;
+        if (h >= sh.extra[xcd]) return;
+        for (unsigned y = 0; y < xcd; y++) h += sh.extra[y];          // position in the list of donated tiles
+        owner = 8;
+        for (unsigned d = 0; d < 8; d++) {
+            const int given = own - sh.cut[d];
+            if (owner == 8 && h < given) { owner = d; slot = sh.cut[d] + h; }
+            if (owner == 8) h -= given;
+        }
+        if (owner == 8) return;
+    } else if (slot >= sh.cut[xcd]) {
+        return;                                                       // donated away
+    }
+    const unsigned uslot = (unsigned)slot;
+    const long long tile = ((((long long)(uslot >> r) << 3) + owner) << r) + (uslot & ((1u << r) - 1u));
+    const long long i = tile * 256 + tid;
+    const v4i v = ld<true>(src + i);
+    st<true>(dst + i, v);
+    if (stamps && tid == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        stamps[2 * (size_t)blockIdx.x + 1] = wall_clock64();
+    }
+}
+
 // A fixed grid; workgroup b takes chunks b, b + grid, b + 2 grid, ... of K * blockDim.x vectors
 // (dst == nullptr: read only; src == nullptr: write only).
 // All K loads of a chunk are complete before its first store is issued, so each workgroup
@@ -191,6 +230,34 @@ int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block,
     }
     hipLaunchKernelGGL(fn, dim3((unsigned)tiles), dim3(block), 0, stream, (v4i*)dst, (const v4i*)src,
                        (unsigned)stripe_log2, flags, sink, stamps);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
+}
+
+// The nt copy, one workgroup per 4 KiB, with per-XCD shares: XCD x does cut[x] of its own tiles plus
+// extra[x] of the tiles the others leave over (the sum of own - cut must equal the sum of extra).
+// `stamps`: null, or two device words per workgroup slot of the grid, 8 * (own + max extra).
+int hbm_ceiling_balanced_copy(void* dst, const void* src, size_t bytes, int stripe_log2, const int* cut, const int* extra,
+                              unsigned long long* stamps, hipStream_t stream) {
+    if (stripe_log2 < 0 || stripe_log2 > 12) return fail("stripe_log2 must be in 0..12");
+    if (!dst || !src || !cut || !extra) return fail("null argument");
+    const size_t period = ((size_t)4096 * 8) << stripe_log2;
+    if (bytes == 0 || bytes % period) return fail("bytes must be a whole number of 8-XCD stripe periods");
+    const long long own = (long long)(bytes / 4096 / 8);
+    xcd_shares sh;
+    long long given = 0, taken = 0, most = 0;
+    for (int x = 0; x < 8; x++) {
+        if (cut[x] < 0 || cut[x] > own || extra[x] < 0 || (extra[x] > 0 && cut[x] != own)) return fail("bad shares");
+        sh.cut[x] = cut[x];
+        sh.extra[x] = extra[x];
+        given += own - cut[x];
+        taken += extra[x];
+        most = extra[x] > most ? extra[x] : most;
+    }
+    if (given != taken) return fail("donated and taken tiles differ");
+    if ((own + most) * 8 > 0x7fffffffll) return fail("too many workgroups");
+    hipLaunchKernelGGL(balanced_copy_kernel, dim3((unsigned)((own + most) * 8)), dim3(256), 0, stream, (v4i*)dst,
+                       (const v4i*)src, (unsigned)stripe_log2, (int)own, sh, stamps);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
 }

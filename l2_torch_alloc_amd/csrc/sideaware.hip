@@ -796,6 +796,11 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
 void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideaware_segment* segments,
                                  int device, sideaware_stream_t stream) {
     if (num_segments <= 0 || !segments) return;
+    bool any_work = false;
+    for (int i = 0; i < num_segments && !any_work; i++) {
+        any_work = segments[i].num_bytes != 0 && (segments[i].out[0] != nullptr || segments[i].in[0] != nullptr);
+    }
+    if (!any_work) return;                       // as a single launch of nothing would (sideaware.cu:1366)
     DeviceContext* ctx = get_context(device);
     if (!ctx) return;
     const Tuning t = tuning_snapshot();

@@ -84,6 +84,11 @@ def test_zero_byte_and_null_calls_return_before_touching_a_device(lib):
     lib.sideaware_memcpy(0, 0, 0, 0, None)
     lib.sideaware_memcpy(0, 0, 4096, 0, None)          # both pointers null
     lib.sideaware_free_auto(None, 0, 0, None)
+    lib.sideaware_elementwise_batch(0, 0, None, 0, None)
+    from l2_torch_alloc_amd import ops
+    empty = (ops._Segment * 3)()                       # three segments, none with anything to do
+    empty[1].num_bytes = 4096                          # bytes but no pointers
+    lib.sideaware_elementwise_batch(0, 3, empty, 0, None)
     assert lib.sideaware_last_error() == b""
 
 

@@ -111,6 +111,25 @@ def test_batched_copy_matches_the_sources(sa):
     assert lib.sideaware_last_error() == b""
 
 
+def test_batched_launch_refuses_a_misaligned_segment_and_runs_nothing(sa):
+    lib = sa.library()
+    from l2_torch_alloc_amd import ops
+    src = torch.randint(1, 256, (2 * MiB,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(2 * MiB, dtype=torch.uint8, device="cuda")
+    arr = (ops._Segment * 2)()
+    arr[0].num_bytes, arr[0].out[0], arr[0].inp[0] = MiB, dst.data_ptr(), src.data_ptr()
+    arr[1].num_bytes, arr[1].out[0], arr[1].inp[0] = 4096, dst.data_ptr() + MiB + 8, src.data_ptr() + MiB      # 8-byte aligned only
+    lib.sideaware_clear_error()
+    lib.sideaware_elementwise_batch(0, 2, arr, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert "multiples of 16" in sa.sideaware_last_error()
+    assert int(dst.sum()) == 0                           # the good segment did not run either: all or nothing per launch
+    lib.sideaware_clear_error()
+    lib.sideaware_elementwise_batch(99999, 1, arr, 0, torch.cuda.current_stream().cuda_stream)
+    assert "never created" in sa.sideaware_last_error()
+    lib.sideaware_clear_error()
+
+
 # --------------------------------------------------------------------------------------- RoPE, q and k in one launch
 
 def test_rope_q_and_k_in_one_launch_vs_oracle(sa):
