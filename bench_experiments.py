@@ -183,6 +183,8 @@ def ceiling_library():
     vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     lib.hbm_ceiling_tile.argtypes = [vp, vp, sz, ci, ci, ci, ci, vp, vp, vp]
     lib.hbm_ceiling_tile.restype = ci
+    lib.hbm_ceiling_policy.argtypes = [vp, vp, sz, ci, ctypes.c_char_p, ctypes.c_char_p, ci, vp, vp]
+    lib.hbm_ceiling_policy.restype = ci
     lib.hbm_ceiling_balanced_copy.argtypes = [vp, vp, sz, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), vp, vp]
     lib.hbm_ceiling_balanced_copy.restype = ci
     lib.hbm_ceiling_persistent.argtypes = [vp, vp, sz, ci, ci, ci, ci, ctypes.c_uint, vp, vp]
@@ -314,6 +316,24 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
                 out[name] = {"us": round(sec * 1e6, 2), "GBps": round(gbps(2 * size, sec), 1)}
                 log("%-58s %9.1f us %8.1f GB/s" % (name, sec * 1e6, gbps(2 * size, sec)))
         del big_src, big_dst
+    # the cache-policy bits of loads and stores, spelled out in the instructions
+    if only and any("policy bits" in o for o in only):
+        bits = ("", "nt", "sc1", "sc0 sc1", "sc1 nt", "sc0 sc1 nt", "sc0")
+        r = 8 if nbytes >= 512 * MiB else 5
+
+        def policy(loads, stores, mode):
+            def launch(d, s_):
+                return ceil.hbm_ceiling_policy(d, s_, nbytes, r, loads.encode(), stores.encode(), mode, sink.data_ptr(), stream)
+            return launch
+
+        for rnd in range(2):
+            for lb in bits:
+                run("policy bits: read-only, loads '%s' (round %d)" % (lb, rnd), nbytes, policy(lb, "", 1))
+            for sb in bits:
+                run("policy bits: write-only, stores '%s' (round %d)" % (sb, rnd), nbytes, policy("", sb, 2))
+            for lb in bits:
+                for sb in bits:
+                    run("policy bits: copy, loads '%s', stores '%s' (round %d)" % (lb, sb, rnd), 2 * nbytes, policy(lb, sb, 0))
     # unequal shares per XCD: measure how far ahead of the last XCD each one finishes, give the slow
     # ones fewer tiles and the fast ones more, and time the copy again
     if only and any("xcd shares" in o for o in only):

@@ -89,6 +89,127 @@ __global__ __launch_bounds__(1024) void tile_kernel(v4i* dst, const v4i* src, un
     }
 }
 
+// The one-workgroup-per-4-KiB kernel with the cache-policy bits of its loads and stores spelled out
+// in the instruction (sc0 / sc1: the scope the access is coherent at, workgroup / agent / both:
+// system; nt: nontemporal).  mode 0: copy, 1: read only, 2: write only.
+#define POLICY_KERNEL(NAME, LOADP, STOREP)                                                                   \
+    __global__ __launch_bounds__(256) void NAME(v4i* dst, const v4i* src, unsigned r, int mode, int* sink) {  \
+        const long long i = striped_tile(blockIdx.x, r) * 256 + threadIdx.x;                                  \
+        v4i v = (v4i){(int)threadIdx.x, 1, (int)blockIdx.x, 7};                                               \
+        if (mode != 2) {                                                                                      \
+            const v4i* p = src + i;                                                                           \
+            asm volatile("global_load_dwordx4 %0, %1, off " LOADP "\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory"); \
+        }                                                                                                     \
+        if (mode != 1) {                                                                                      \
+            v4i* q = dst + i;                                                                                 \
+            asm volatile("global_store_dwordx4 %0, %1, off " STOREP "\n\ts_nop 1" : : "v"(q), "v"(v) : "memory"); \
+        } else {                                                                                              \
+            sink_if_magic(v, sink);                                                                           \
+        }                                                                                                     \
+    }
+POLICY_KERNEL(policy_plain_plain, "", "")
+POLICY_KERNEL(policy_plain_nt, "", "nt")
+POLICY_KERNEL(policy_plain_sc1, "", "sc1")
+POLICY_KERNEL(policy_plain_sc0sc1, "", "sc0 sc1")
+POLICY_KERNEL(policy_plain_sc1nt, "", "sc1 nt")
+POLICY_KERNEL(policy_plain_sc0sc1nt, "", "sc0 sc1 nt")
+POLICY_KERNEL(policy_plain_sc0, "", "sc0")
+POLICY_KERNEL(policy_nt_plain, "nt", "")
+POLICY_KERNEL(policy_nt_nt, "nt", "nt")
+POLICY_KERNEL(policy_nt_sc1, "nt", "sc1")
+POLICY_KERNEL(policy_nt_sc0sc1, "nt", "sc0 sc1")
+POLICY_KERNEL(policy_nt_sc1nt, "nt", "sc1 nt")
+POLICY_KERNEL(policy_nt_sc0sc1nt, "nt", "sc0 sc1 nt")
+POLICY_KERNEL(policy_nt_sc0, "nt", "sc0")
+POLICY_KERNEL(policy_sc1_plain, "sc1", "")
+POLICY_KERNEL(policy_sc1_nt, "sc1", "nt")
+POLICY_KERNEL(policy_sc1_sc1, "sc1", "sc1")
+POLICY_KERNEL(policy_sc1_sc0sc1, "sc1", "sc0 sc1")
+POLICY_KERNEL(policy_sc1_sc1nt, "sc1", "sc1 nt")
+POLICY_KERNEL(policy_sc1_sc0sc1nt, "sc1", "sc0 sc1 nt")
+POLICY_KERNEL(policy_sc1_sc0, "sc1", "sc0")
+POLICY_KERNEL(policy_sc0sc1_plain, "sc0 sc1", "")
+POLICY_KERNEL(policy_sc0sc1_nt, "sc0 sc1", "nt")
+POLICY_KERNEL(policy_sc0sc1_sc1, "sc0 sc1", "sc1")
+POLICY_KERNEL(policy_sc0sc1_sc0sc1, "sc0 sc1", "sc0 sc1")
+POLICY_KERNEL(policy_sc0sc1_sc1nt, "sc0 sc1", "sc1 nt")
+POLICY_KERNEL(policy_sc0sc1_sc0sc1nt, "sc0 sc1", "sc0 sc1 nt")
+POLICY_KERNEL(policy_sc0sc1_sc0, "sc0 sc1", "sc0")
+POLICY_KERNEL(policy_sc1nt_plain, "sc1 nt", "")
+POLICY_KERNEL(policy_sc1nt_nt, "sc1 nt", "nt")
+POLICY_KERNEL(policy_sc1nt_sc1, "sc1 nt", "sc1")
+POLICY_KERNEL(policy_sc1nt_sc0sc1, "sc1 nt", "sc0 sc1")
+POLICY_KERNEL(policy_sc1nt_sc1nt, "sc1 nt", "sc1 nt")
+POLICY_KERNEL(policy_sc1nt_sc0sc1nt, "sc1 nt", "sc0 sc1 nt")
+POLICY_KERNEL(policy_sc1nt_sc0, "sc1 nt", "sc0")
+POLICY_KERNEL(policy_sc0sc1nt_plain, "sc0 sc1 nt", "")
+POLICY_KERNEL(policy_sc0sc1nt_nt, "sc0 sc1 nt", "nt")
+POLICY_KERNEL(policy_sc0sc1nt_sc1, "sc0 sc1 nt", "sc1")
+POLICY_KERNEL(policy_sc0sc1nt_sc0sc1, "sc0 sc1 nt", "sc0 sc1")
+POLICY_KERNEL(policy_sc0sc1nt_sc1nt, "sc0 sc1 nt", "sc1 nt")
+POLICY_KERNEL(policy_sc0sc1nt_sc0sc1nt, "sc0 sc1 nt", "sc0 sc1 nt")
+POLICY_KERNEL(policy_sc0sc1nt_sc0, "sc0 sc1 nt", "sc0")
+POLICY_KERNEL(policy_sc0_plain, "sc0", "")
+POLICY_KERNEL(policy_sc0_nt, "sc0", "nt")
+POLICY_KERNEL(policy_sc0_sc1, "sc0", "sc1")
+POLICY_KERNEL(policy_sc0_sc0sc1, "sc0", "sc0 sc1")
+POLICY_KERNEL(policy_sc0_sc1nt, "sc0", "sc1 nt")
+POLICY_KERNEL(policy_sc0_sc0sc1nt, "sc0", "sc0 sc1 nt")
+POLICY_KERNEL(policy_sc0_sc0, "sc0", "sc0")
+
+typedef void (*policy_fn)(v4i*, const v4i*, unsigned, int, int*);
+static const struct { const char* loads; const char* stores; policy_fn fn; } kPolicyKernels[] = {
+    {"", "", policy_plain_plain},
+    {"", "nt", policy_plain_nt},
+    {"", "sc1", policy_plain_sc1},
+    {"", "sc0 sc1", policy_plain_sc0sc1},
+    {"", "sc1 nt", policy_plain_sc1nt},
+    {"", "sc0 sc1 nt", policy_plain_sc0sc1nt},
+    {"", "sc0", policy_plain_sc0},
+    {"nt", "", policy_nt_plain},
+    {"nt", "nt", policy_nt_nt},
+    {"nt", "sc1", policy_nt_sc1},
+    {"nt", "sc0 sc1", policy_nt_sc0sc1},
+    {"nt", "sc1 nt", policy_nt_sc1nt},
+    {"nt", "sc0 sc1 nt", policy_nt_sc0sc1nt},
+    {"nt", "sc0", policy_nt_sc0},
+    {"sc1", "", policy_sc1_plain},
+    {"sc1", "nt", policy_sc1_nt},
+    {"sc1", "sc1", policy_sc1_sc1},
+    {"sc1", "sc0 sc1", policy_sc1_sc0sc1},
+    {"sc1", "sc1 nt", policy_sc1_sc1nt},
+    {"sc1", "sc0 sc1 nt", policy_sc1_sc0sc1nt},
+    {"sc1", "sc0", policy_sc1_sc0},
+    {"sc0 sc1", "", policy_sc0sc1_plain},
+    {"sc0 sc1", "nt", policy_sc0sc1_nt},
+    {"sc0 sc1", "sc1", policy_sc0sc1_sc1},
+    {"sc0 sc1", "sc0 sc1", policy_sc0sc1_sc0sc1},
+    {"sc0 sc1", "sc1 nt", policy_sc0sc1_sc1nt},
+    {"sc0 sc1", "sc0 sc1 nt", policy_sc0sc1_sc0sc1nt},
+    {"sc0 sc1", "sc0", policy_sc0sc1_sc0},
+    {"sc1 nt", "", policy_sc1nt_plain},
+    {"sc1 nt", "nt", policy_sc1nt_nt},
+    {"sc1 nt", "sc1", policy_sc1nt_sc1},
+    {"sc1 nt", "sc0 sc1", policy_sc1nt_sc0sc1},
+    {"sc1 nt", "sc1 nt", policy_sc1nt_sc1nt},
+    {"sc1 nt", "sc0 sc1 nt", policy_sc1nt_sc0sc1nt},
+    {"sc1 nt", "sc0", policy_sc1nt_sc0},
+    {"sc0 sc1 nt", "", policy_sc0sc1nt_plain},
+    {"sc0 sc1 nt", "nt", policy_sc0sc1nt_nt},
+    {"sc0 sc1 nt", "sc1", policy_sc0sc1nt_sc1},
+    {"sc0 sc1 nt", "sc0 sc1", policy_sc0sc1nt_sc0sc1},
+    {"sc0 sc1 nt", "sc1 nt", policy_sc0sc1nt_sc1nt},
+    {"sc0 sc1 nt", "sc0 sc1 nt", policy_sc0sc1nt_sc0sc1nt},
+    {"sc0 sc1 nt", "sc0", policy_sc0sc1nt_sc0},
+    {"sc0", "", policy_sc0_plain},
+    {"sc0", "nt", policy_sc0_nt},
+    {"sc0", "sc1", policy_sc0_sc1},
+    {"sc0", "sc0 sc1", policy_sc0_sc0sc1},
+    {"sc0", "sc1 nt", policy_sc0_sc1nt},
+    {"sc0", "sc0 sc1 nt", policy_sc0_sc0sc1nt},
+    {"sc0", "sc0", policy_sc0_sc0},
+};
+
 // The one-workgroup-per-4-KiB nt copy with unequal shares per XCD.  Workgroups are dealt to the
 // XCDs in turn, so each XCD gets the same number of workgroup slots (own + the largest extra);
 // XCD x does only the first cut[x] of its own tiles, and the tiles the donors leave over are done
@@ -232,6 +353,26 @@ int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block,
                        (unsigned)stripe_log2, flags, sink, stamps);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
+}
+
+// One workgroup per 4 KiB with the given cache-policy bits on loads and stores ("", "nt", "sc1",
+// "sc0 sc1", "sc1 nt", "sc0 sc1 nt", "sc0").  mode 0: copy, 1: read only, 2: write only.
+int hbm_ceiling_policy(void* dst, const void* src, size_t bytes, int stripe_log2, const char* loads, const char* stores,
+                       int mode, int* sink, hipStream_t stream) {
+    if (stripe_log2 < 0 || stripe_log2 > 12) return fail("stripe_log2 must be in 0..12");
+    if (!loads || !stores || !sink || mode < 0 || mode > 2) return fail("bad argument");
+    if ((mode != 2 && !src) || (mode != 1 && !dst)) return fail("null buffer");
+    const size_t period = ((size_t)4096 * 8) << stripe_log2;
+    if (bytes == 0 || bytes % period || bytes / 4096 > 0x7fffffffull) return fail("bytes must be a whole number of 8-XCD stripe periods");
+    for (const auto& k : kPolicyKernels) {
+        if (std::strcmp(k.loads, loads) == 0 && std::strcmp(k.stores, stores) == 0) {
+            hipLaunchKernelGGL(k.fn, dim3((unsigned)(bytes / 4096)), dim3(256), 0, stream, (v4i*)dst, (const v4i*)src,
+                               (unsigned)stripe_log2, mode, sink);
+            hipError_t e = hipGetLastError();
+            return e == hipSuccess ? 0 : fail(hipGetErrorString(e));
+        }
+    }
+    return fail("no kernel with these policy bits");
 }
 
 // The nt copy, one workgroup per 4 KiB, with per-XCD shares: XCD x does cut[x] of its own tiles plus

@@ -281,11 +281,12 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     assert loads and stores
     assert all(" nt" in l for l in loads), loads            # read once: nontemporal
     assert not any(" nt" in s for s in stores), stores        # fits the Infinity Cache: kept for the consumer
+    assert all(" sc1" in s for s in stores), stores           # written through the private L2 (agent scope)
     # in place (variant bit 2) with an evict-marked input: the stores stream as well
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 4), "sideaware_copy")
     assert all(" nt" in l for l in loads) and all(" nt" in s for s in stores)
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 2), "sideaware_copy")
-    assert all(" nt" in l for l in loads) and all(" nt" in s for s in stores)   # larger: everything streams
+    assert all(" nt" in l for l in loads) and all(" nt" in s and " sc1" in s for s in stores)   # larger: everything streams
     # RoPE: the activations stream, the gathered table never does
     rope = headers.rope_header(4096, 32, 0, 128, "bf16", "heads", unrolled=1)
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, rope, 2),
@@ -296,7 +297,16 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     fixed = headers.rope_header(4096, 32, 0, 128, "bf16", "heads", unrolled=1, stream_output=False)
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, fixed, 4),
                                 "sideaware_rope_fwd_bf16_heads_t4096_h32_0_d128")
-    assert stores and not any(" nt" in s for s in stores)
+    assert stores and not any(" nt" in s for s in stores) and all(" sc1" in s for s in stores)
+    # an expert header names the bits of its 16-byte stores itself
+    expert = b'#define SA_STORE_POLICY "sc0 sc1 nt"\n' + headers.memcpy_header()
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, expert, 0), "sideaware_copy_spelled_out")
+    assert stores and all(" sc0" in s and " sc1" in s and " nt" in s for s in stores), stores
+    # narrower outputs get the same policy on their narrower stores
+    mixed = headers.mxfp8_quantize_header()            # bf16 in (16 B per lane), fp8 out (8 B per lane)
+    body = _isa_of(lib, tmp_path, mixed, 0)
+    narrow = [l for l in body.splitlines() if "global_store_dwordx2" in l]
+    assert narrow and all(" sc1" in l for l in narrow), narrow
     # bf16 is narrowed by the hardware's round-to-nearest-even convert, fp32 math is not fused
     isa = _isa_of(lib, tmp_path, rope, 0)
     assert "v_cvt_pk_bf16_f32" in isa and "v_fma_f32" not in isa and "v_pk_mul_f32" not in isa
@@ -335,3 +345,21 @@ def test_damaged_cache_files_read_as_misses(lib, tmp_path, monkeypatch):
         files[0].write_bytes(damaged)
         assert compile_ok(lib, header, 0)[0] == 0
         assert files[0].read_bytes() == good                    # rebuilt: same source, same code object
+
+
+def test_every_wide_store_is_followed_by_two_wait_states(lib, tmp_path):
+    # The 16-byte stores are written as instructions, which the compiler's hazard pass does not
+    # look into: the hardware reads a wide store's data registers for two more issue cycles, so
+    # each such store must be followed by `s_nop 1` before the compiler's next instruction (which
+    # may overwrite them).  Checked over the size / alignment classes and both entry points.
+    hn = headers.rope_header(4096, 0, 0, 128, "bf16", "heads", heads_at_launch=True)
+    fixed = headers.rope_header(4096, 32, 0, 128, "bf16", "heads")
+    seen = 0
+    for header, variant in ((None, 0), (None, 2), (None, 3), (None, 12), (hn, 4), (hn, 2), (fixed, 4), (fixed, 10)):
+        lines = [l.strip() for l in _isa_of(lib, tmp_path, header, variant).splitlines()]
+        lines = [l.split("//")[0].strip() for l in lines if l and not l.startswith(("//", ";"))]
+        for i, l in enumerate(lines):
+            if l.startswith("global_store_dwordx4") or l.startswith("global_store_dwordx3"):
+                seen += 1
+                assert lines[i + 1].startswith("s_nop 1"), (variant, lines[i:i + 3])
+    assert seen >= 16
