@@ -38,7 +38,8 @@ def stripe_ab(steps):
 def chain_policy(reps=6):
     """The evidence behind the cache-policy classes: a producer launch followed at once by a consumer
     that reads its result (this library's copy), over buffer sets that cycle so that nothing is
-    cache-resident, with the producer's stores plain or nontemporal.  Producers: a copy (not in
+    cache-resident, with the producer's stores left cacheable ("plain": OUTPUT_STREAMING 0) or
+    streaming ("nt": OUTPUT_STREAMING 1).  Producers: a copy (not in
     place) and the bf16 RoPE (in place), at several sizes.  Per-launch times from HIP events."""
     import torch
     from l2_torch_alloc_amd import headers, ops, wrapper
@@ -593,20 +594,25 @@ def launch_shapes(steps, only=None):
 
 def chain_xcd(reps=4, only=None):
     """Producer -> consumer on the same buffer, meant to be run under `rocprofv3 --pmc` with the per-XCD
-    TCC_HIT / TCC_MISS counters of profiles/xcd_counters.yaml: a copy writes `mid` (stores plain or
-    nontemporal), and at once a second copy reads `mid`, walking each XCD's tiles in the same order
-    or in reverse (`reverse_order`, the reference's knob for exactly this: sideaware.cu:40), so that
-    it starts with what the producer wrote last.  Buffer sets cycle, so nothing but the producer's
-    result can be cache-resident.  Kernel names carry size, store policy and order; per-launch times
-    come from HIP events."""
+    TCC_HIT / TCC_MISS counters of profiles/xcd_counters.yaml: a copy writes `mid`, and at once a
+    second copy reads `mid`, walking each XCD's tiles in the same order or in reverse
+    (`reverse_order`, the reference's knob for exactly this: sideaware.cu:40), so that it starts with
+    what the producer wrote last.  The producer's stores are the library's two policies, `sc1`
+    (written through the private L2, left cacheable) and `sc1nt` (the same, streaming), or, for
+    comparison, the same stores without the scope bit (`plain`, `nt`).  Buffer sets cycle, so nothing
+    but the producer's result can be cache-resident.  Kernel names carry size, store policy and
+    order; per-launch times come from HIP events."""
     import torch
     from l2_torch_alloc_amd import headers, wrapper
     lib, stream = _abi()
     base = headers.memcpy_header().decode()
     out = {}
 
-    def kernel(tag, stream_out, reverse, stream_in=1):
-        text = "#define INPUT0_STREAMING %d\n#define OUTPUT_STREAMING %d\n" % (stream_in, stream_out) + base
+    store_defines = {"sc1": "#define OUTPUT_STREAMING 0\n", "sc1nt": "#define OUTPUT_STREAMING 1\n",
+                     "plain": '#define SA_STORE_POLICY ""\n', "nt": '#define SA_STORE_POLICY "nt"\n'}
+
+    def kernel(tag, stores, reverse, stream_in=1):
+        text = "#define INPUT0_STREAMING %d\n" % stream_in + store_defines[stores] + base
         text = text.replace("#define KERNEL_NAME ", "#define KERNEL_NAME " + tag)
         text = text.replace("constexpr bool reverse_order = false;", "constexpr bool reverse_order = %s;" % ("true" if reverse else "false"))
         return wrapper.sideaware_create_kernel(text.encode())
@@ -618,15 +624,15 @@ def chain_xcd(reps=4, only=None):
         mids = [torch.empty_like(t) for t in srcs]
         outs = [torch.empty_like(t) for t in srcs]
         # the consumer's loads carry the streaming hint, except in the "plainloads" cases
-        cases = [(policy, order, 1) for policy in ("plain", "nt") for order in ("same", "reversed")]
-        cases += [("plain", "same", 0), ("plain", "reversed", 0)]
+        cases = [(policy, order, 1) for policy in ("sc1", "sc1nt") for order in ("same", "reversed")]
+        cases += [("plain", "same", 1), ("nt", "same", 1), ("sc1", "same", 0), ("sc1", "reversed", 0)]
         for policy, order, consumer_stream_in in cases:
-                stream_out, reverse = int(policy == "nt"), order == "reversed"
+                reverse = order == "reversed"
                 name = "%dMiB_%s_%s%s" % (mib, policy, order, "" if consumer_stream_in else "_plainloads")
                 if only and not any(o in name for o in only):
                     continue
-                producer = kernel("chainP_%s_" % name, stream_out, False)
-                consumer = kernel("chainC_%s_" % name, 1, reverse, consumer_stream_in)
+                producer = kernel("chainP_%s_" % name, policy, False)
+                consumer = kernel("chainC_%s_" % name, "sc1nt", reverse, consumer_stream_in)
                 evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(sets)]
                 tp = tc = 0.0
                 for rep in range(reps + 1):
