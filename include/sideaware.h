@@ -142,9 +142,10 @@ const char* sideaware_last_error(void);
 void sideaware_clear_error(void);
 /* Compiles header + template for gfx950 without touching a device. variant bit 0: 0 = 32-bit indices
  * (arrays below 2 GiB), 1 = 64-bit indices; bit 1: 0 = the array fits the Infinity Cache
- * (outputs written plainly), 1 = larger (everything streams); bit 2: 1 = o0 is written over i0
+ * (outputs left cacheable), 1 = larger (everything streams); bit 2: 1 = o0 is written over i0
  * (in place: outputs stream when i0 is marked input_evict); bit 3: 1 = i0 or o0 is not 2 MiB-aligned
- * (`aligned_2MiB` is false, as it is with 64-bit indices).  Returns 0 on success; the compiler
+ * (`aligned_2MiB` is false, as it is with 64-bit indices); bit 4: 1 = an output does not start on
+ * a 64-byte boundary (write-back stores instead of write-through ones).  Returns 0 on success; the compiler
  * log (possibly empty) is copied to `log`. */
 int sideaware_compile_check(const char* header, int variant, char* log, size_t log_capacity);
 /* The kernel template and the built-in copy header, as compiled (for audits and CPU harnesses). */

@@ -302,6 +302,14 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     expert = b'#define SA_STORE_POLICY "sc0 sc1 nt"\n' + headers.memcpy_header()
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, expert, 0), "sideaware_copy_spelled_out")
     assert stores and all(" sc0" in s and " sc1" in s and " nt" in s for s in stores), stores
+    # an output that does not start on a 64-byte boundary (variant bit 4): the compiler's stores,
+    # which the L2 may merge; streaming ones where the aligned launch would stream
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 16), "sideaware_copy")
+    assert stores and not any(" sc1" in s or " nt" in s for s in stores), stores
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 16 | 2), "sideaware_copy")
+    assert stores and all(" nt" in s and " sc1" not in s for s in stores), stores
+    loads, stores = _memory_ops(_isa_of(lib, tmp_path, expert, 16), "sideaware_copy_spelled_out")
+    assert stores and all(" sc0" in s and " sc1" in s and " nt" in s for s in stores), stores   # an expert's bits stand
     # narrower outputs get the same policy on their narrower stores
     mixed = headers.mxfp8_quantize_header()            # bf16 in (16 B per lane), fp8 out (8 B per lane)
     body = _isa_of(lib, tmp_path, mixed, 0)

@@ -111,6 +111,35 @@ def test_batched_copy_matches_the_sources(sa):
     assert lib.sideaware_last_error() == b""
 
 
+@pytest.mark.parametrize("nbytes", [4096 + 16, 8 * MiB + 48, 300 * MiB])
+@pytest.mark.parametrize("offset", [16, 48, 80])
+def test_copy_to_a_destination_off_a_64_byte_boundary(sa, nbytes, offset):
+    # such a launch takes the instantiation with write-back stores (its store instructions cover
+    # pieces of memory lines); same bytes, nothing outside them, in both cache classes and in place
+    lib = sa.library()
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+    dst = torch.full((nbytes + 512,), 0x5A, dtype=torch.uint8, device="cuda")
+    assert dst.data_ptr() % 64 == 0 and src.data_ptr() % 64 == 0
+    lib.sideaware_memcpy(dst.data_ptr() + offset, src.data_ptr(), nbytes, 0, stream)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert torch.equal(dst[offset:offset + nbytes], src)
+    assert bool((dst[:offset] == 0x5A).all()) and bool((dst[offset + nbytes:] == 0x5A).all())
+    if nbytes <= 8 * MiB + 48:
+        # in place at the same odd offset: bf16 scale+bias over the copied bytes against the oracle
+        from l2_torch_alloc_amd import ops
+        n = (nbytes // 16) * 8
+        x = dst[offset:offset + 2 * n].view(torch.bfloat16)
+        x.copy_(torch.randn(n, device="cuda").to(torch.bfloat16))
+        before = bits(x).copy()
+        ops.scale_bias_bf16(x, torch.tensor([1.5, -0.25], dtype=torch.float32, device="cuda"), out=x)
+        torch.cuda.synchronize()
+        assert_no_library_error(sa)
+        assert np.array_equal(bits(x), O.scale_bias_bf16(before, 1.5, -0.25))
+        assert bool((dst[:offset] == 0x5A).all()) and bool((dst[offset + nbytes:] == 0x5A).all())
+
+
 def test_batched_launch_refuses_a_misaligned_segment_and_runs_nothing(sa):
     lib = sa.library()
     from l2_torch_alloc_amd import ops
