@@ -116,7 +116,7 @@ def bench_copy_cold(nbytes, steps):
             "after_read_scrub": {"us_median": clean * 1e6, "GBps": gbps(2 * nbytes, clean)}}
 
 
-def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0):
+def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
     """The headline protocol.  `steps` back-to-back launches that cycle through `pairs` distinct
     (src, dst) pairs, so no launch finds an operand in a cache (the working set is
     pairs * 2 * nbytes, far beyond the 256 MB Infinity Cache) and the only dirty lines in its way
@@ -137,8 +137,8 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0):
         counter[0] += 1
         lib.sideaware_memcpy(d_ptr, s_ptr, nbytes, 0, stream)
 
-    for _ in range(pairs):                       # every destination is written at least once
-        launch()
+    for _ in range(pairs + prewarm):             # every destination is written at least once; the
+        launch()                                 # rest brings the device to its steady clocks
     sec = time_region(launch, steps, warmup)
     ok = all(bool(torch.equal(d, t)) for d, t in zip(dsts, srcs))
     return {"bytes": nbytes, "pairs": pairs, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec),
@@ -238,7 +238,7 @@ def bench_energy(seconds=2.5):
     return out
 
 
-def bench_rope_bf16(steps, warmup, main_figure_only=False):
+def bench_rope_bf16(steps, warmup, main_figure_only=False, prewarm=0):
     """q (8,4096,32,128) and k (8,4096,8,128) bf16 in place, fp32 table theta=5e5.  One step rotates
     q and k.  The main figure cycles over five distinct (q, k) sets, so that no tensor is
     cache-resident, with q and k sharing one launch (sideaware_elementwise_batch); the same step as
@@ -291,7 +291,7 @@ def bench_rope_bf16(steps, warmup, main_figure_only=False):
         launch_q(a.data_ptr())
         launch_k(b.data_ptr())
 
-    sec = time_region(step_one_launch, steps, warmup + sets)
+    sec = time_region(step_one_launch, steps, warmup + sets + prewarm)
     main = {"bytes": total, "us": sec * 1e6, "GBps": gbps(total, sec), "frac_of_peak": gbps(total, sec) / HBM_PEAK_GBPS,
             "protocol": "steps cycle over five distinct (q, k) sets (1.6 GB): no tensor is cache-resident; "
                         "q and k share one launch"}
@@ -401,6 +401,22 @@ def bench_churn(use_sideaware, n_ops=10000, live_cap=64 * GiB):
         from l2_torch_alloc_amd import ops
         sb = torch.tensor([1.5, 0.25], dtype=torch.float32, device="cuda")
     sizes = churn_sizes(n_ops)
+
+    def op(x, y):
+        if use_sideaware:
+            ops.scale_bias_bf16(x, sb, out=y)
+        else:
+            torch.add(x * 1.5, 0.25, out=y)
+
+    # Untimed: one op per size and alignment class, so that no first-use compile (the library
+    # builds an instantiation per class on first use) or lazy initialisation of PyTorch's kernels
+    # falls between the events of a sampled op below.
+    for size in (4096, 3 * MiB + 4096, 64 * MiB, 300 * MiB):
+        pad = torch.empty(size // 2 + 256, dtype=torch.bfloat16, device="cuda")
+        for x in (torch.empty(size // 2, dtype=torch.bfloat16, device="cuda"), pad[256:]):
+            op(x.normal_(), torch.empty_like(x))
+        del pad, x
+    torch.cuda.synchronize()
     live, live_bytes = [], 0
     t_alloc, t_free = [], []
     op_bytes, op_seconds = 0, 0.0
@@ -415,10 +431,7 @@ def bench_churn(use_sideaware, n_ops=10000, live_cap=64 * GiB):
         y = torch.empty(n, dtype=torch.bfloat16, device="cuda")
         x.normal_()
         ev0.record()
-        if use_sideaware:
-            ops.scale_bias_bf16(x, sb, out=y)
-        else:
-            torch.add(x * 1.5, 0.25, out=y)
+        op(x, y)
         ev1.record()
         if i % 50 == 0 or size >= 64 * MiB:
             torch.cuda.synchronize()
@@ -556,6 +569,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--prewarm", type=int, default=300,
+                    help="untimed launches of the same protocol ahead of the warmup steps of the two headline figures: "
+                         "the device reaches its steady clocks only after some tens of milliseconds of load")
     ap.add_argument("--quick", action="store_true", help="the two headline protocols (copy, bf16 RoPE) and the CPU baseline only")
     ap.add_argument("--stripe-ab", action="store_true",
                     help="only the stripe-size A/B of the q RoPE (for a FETCH_SIZE profile)")
@@ -620,11 +636,11 @@ def main():
         print(json.dumps({"ceiling": experiments.ceiling(args.steps, only=args.only)}))
         return
 
-    copy = bench_copy_rotating(256 * MiB, 8, args.steps, args.warmup, seed=0)
+    copy = bench_copy_rotating(256 * MiB, 8, args.steps, args.warmup, seed=0, prewarm=args.prewarm)
     log("copy 256 MiB, cycling over 8 pairs:", copy)
     # --quick times the two headline protocols and nothing else of this library, so that a kernel
     # trace of the run holds one protocol per kernel name
-    rope = bench_rope_bf16(args.steps, args.warmup, main_figure_only=args.quick)
+    rope = bench_rope_bf16(args.steps, args.warmup, main_figure_only=args.quick, prewarm=args.prewarm)
     log("rope bf16:", rope)
     also = {"rope_bf16_llama3_8b": rope}
     warm = None
@@ -695,7 +711,8 @@ def main():
         "config": {"workload": "byte memcpy of 256 MiB, uint8 uniform [0,255], seed 0, dst = src "
                                "(2 MiB-aligned regions from the sideaware pool); launches cycle over 8 distinct "
                                "(src, dst) pairs, so no operand is ever cache-resident",
-                   "bit_exact": copy["bit_exact"]},
+                   "bit_exact": copy["bit_exact"],
+                   "untimed_before_warmup": "%d launches of the same cycling protocol (device at steady clocks)" % args.prewarm},
         # Both halves of the metric, each under the protocol in which nothing can be cache-resident.
         # `traffic` is not measured in this run: it is the L2 -> fabric byte count per launch from
         # the rocprofv3 --pmc runs summarised in the named profile.
