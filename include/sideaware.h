@@ -160,8 +160,9 @@ int sideaware_kernel_info(int kernel_id, int variant, int* out);
 /* Pool counters, in the order of struct PoolStats (pool.h); returns the number written. */
 int sideaware_alloc_stats(unsigned long long* out, int capacity);
 /* Tuning knobs: "stripe_bytes" (0 = chosen by array size), "stripes_per_xcd", "slot_run", "groups_cap",
- * "one_shot", "cache_bytes" (launch parameters) and "nt_store", "wg_threads" (compiled in: after a
- * change every op is compiled afresh on its next launch).
+ * "one_shot", "cache_bytes" (launch parameters) and "nt_store", "wg_threads", "write_through"
+ * (1: stores are written through the XCD's private L2; 0: the compiler's write-back stores)
+ * (compiled in: after a change every op is compiled afresh on its next launch).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -90,18 +90,21 @@ struct Tuning {
     long long groups_cap = 8;        // upper bound on default workgroups per CU
     long long wg_threads = 256;
     long long stripes_per_xcd = 8;   // an array gets stripes small enough for every XCD to own at least this many
+    long long write_through = 1;     // 1: stores written through the private L2 (`sc1`); 0: the compiler's write-back stores
 };
 
 // The knobs themselves: written by sideaware_tune (and once from the environment), read by every
 // launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
 // a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
-constexpr int kTuneKnobs = 8;
+constexpr int kTuneKnobs = 9;
 static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
-                                                   "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd"};
+                                                   "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd",
+                                                   "write_through"};
 static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
                                                  "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
-                                                 "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD"};
-static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}};
+                                                 "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD",
+                                                 "SIDEAWARE_WRITE_THROUGH"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -127,6 +130,7 @@ static Tuning tuning_snapshot() {
     t.groups_cap = g_tune[5].load(std::memory_order_relaxed);
     t.wg_threads = g_tune[6].load(std::memory_order_relaxed);
     t.stripes_per_xcd = g_tune[7].load(std::memory_order_relaxed);
+    t.write_through = g_tune[8].load(std::memory_order_relaxed);
     return t;
 }
 
@@ -437,7 +441,8 @@ static std::string config_block(int variant, int num_xcds, int num_cus, const Tu
     s += "#define HASH " + std::to_string((stripe_hash_mask(num_xcds) | (1 << 21)) / 16) + "\n";
     s += "#define SA_BEYOND_CACHE " + std::to_string((variant >> 1) & 1) + "\n";
     s += "#define SA_IN_PLACE " + std::to_string((variant >> 2) & 1) + "\n";
-    s += "#define SA_SPLIT_LINES " + std::to_string((variant >> 4) & 1) + "\n";
+    // the compiler's write-back stores: for outputs off a 64-byte boundary, or when switched to
+    s += "#define SA_SPLIT_LINES " + std::to_string((((variant >> 4) & 1) || !t.write_through) ? 1 : 0) + "\n";
     // As in the reference (sideaware.cu:792-794, 1386-1388): `aligned_2MiB` is true only in the
     // instantiation that launches with 2 MiB-aligned i0 and o0 below 2 GiB are routed to.
     s += (variant & kVariantWide) ? "using size_type = long long;\n" : "using size_type = int;\n";
@@ -1069,7 +1074,8 @@ int sideaware_tune(const char* key, long long value) {
     if (!std::strcmp(key, "stripes_per_xcd") && (value < 1 || value > (1 << 20))) return 1;
     if (slot->load() != value) {
         slot->store(value);
-        const bool compiled_in = !std::strcmp(key, "nt_store") || !std::strcmp(key, "wg_threads");
+        const bool compiled_in = !std::strcmp(key, "nt_store") || !std::strcmp(key, "wg_threads") ||
+                                 !std::strcmp(key, "write_through");
         if (compiled_in) g_tune_generation++;      // compiled kernels are rebuilt on their next use
     }
     return 0;

@@ -256,6 +256,8 @@ def test_reference_rope_header_compiles_unchanged(lib, variant):
 def _isa_of(lib, tmp_path, header, variant):
     """Compiles header + template for gfx950 and returns the disassembly the library wrote."""
     dump = tmp_path / ("isa_%d.txt" % variant)
+    if dump.exists():
+        dump.unlink()                       # the library appends
     lib.sideaware_write_sass(str(dump).encode())
     try:
         rc, log = compile_ok(lib, header, variant)
@@ -310,6 +312,15 @@ def test_cache_policy_is_visible_in_the_isa(lib, tmp_path):
     assert stores and all(" nt" in s and " sc1" not in s for s in stores), stores
     loads, stores = _memory_ops(_isa_of(lib, tmp_path, expert, 16), "sideaware_copy_spelled_out")
     assert stores and all(" sc0" in s and " sc1" in s and " nt" in s for s in stores), stores   # an expert's bits stand
+    # the knob that takes the write-through away: the compiler's stores in every instantiation
+    assert lib.sideaware_tune(b"write_through", 0) == 0
+    try:
+        assert b"#define SA_SPLIT_LINES 1" in lib.sideaware_config_block(0)
+        loads, stores = _memory_ops(_isa_of(lib, tmp_path, None, 0), "sideaware_copy")
+        assert stores and not any(" sc1" in s or " nt" in s for s in stores), stores
+    finally:
+        assert lib.sideaware_tune(b"write_through", 1) == 0
+    assert b"#define SA_SPLIT_LINES 0" in lib.sideaware_config_block(0)
     # narrower outputs get the same policy on their narrower stores
     mixed = headers.mxfp8_quantize_header()            # bf16 in (16 B per lane), fp8 out (8 B per lane)
     body = _isa_of(lib, tmp_path, mixed, 0)
