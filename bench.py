@@ -305,6 +305,14 @@ def bench_rope_bf16(steps, warmup, main_figure_only=False, prewarm=0):
     scrub = torch.empty(GiB, dtype=torch.uint8, device="cuda")
     cold = statistics.median(time_each(lambda: lib.sideaware_elementwise_batch(kid_any, 2, batches[0], 0, stream), 15, 1,
                                        before=lambda: scrub.fill_(1)))
+    # the same step for the half-split pair layout (the partner's vector comes from another lane)
+    kid_half = wrapper.sideaware_create_kernel(headers.rope_half_header(T, 0, HS, "bf16", heads_at_launch=True))
+
+    def step_half():
+        lib.sideaware_elementwise_batch(kid_half, 2, batches[counter[0] % sets], 0, stream)
+        counter[0] += 1
+
+    sec_half = time_region(step_half, steps, warmup + sets)
     del scrub, qk, batches
 
     # for scale: the same step in eager PyTorch (complex multiply in fp32, back to bf16), out of place
@@ -323,6 +331,7 @@ def bench_rope_bf16(steps, warmup, main_figure_only=False, prewarm=0):
                            "note": "1 GiB written over the caches before every step; one event pair per step"},
             "q_only_loop": {"us": sec_q * 1e6, "GBps": gbps(2 * q_bytes + table_bytes, sec_q)},
             "k_only_loop": {"us": sec_k * 1e6, "GBps": gbps(2 * k_bytes + table_bytes, sec_k)},
+            "half_split_pair_layout_same_protocol": {"us": sec_half * 1e6, "GBps": gbps(total, sec_half)},
             "torch_eager_same_step": {"us": sec_torch * 1e6, "GBps_on_the_same_algorithmic_bytes": gbps(total, sec_torch)}}
 
 

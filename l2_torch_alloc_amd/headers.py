@@ -153,6 +153,164 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     return "".join(lines).encode()
 
 
+_ROPE_HALF_TYPES = {
+    # storage dtype -> (element type, elements per 16-byte vector)
+    "fp32": ("float", 4),
+    "bf16": ("__bf16", 8),
+    "fp16": ("_Float16", 8),
+}
+
+
+def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", backward: bool = False,
+                     heads_first: bool = False, heads_at_launch: bool = False, unrolled: int | None = 2,
+                     evict_input: bool = True) -> bytes:
+    """RoPE for the half-split pair layout ("rotate_half": element i of a head is paired with
+    element i + head_dim/2, as Hugging Face / GPT-NeoX style models store q and k), forward or
+    backward, in place or out of place.
+
+    The reference's op (``kernel_rope.cuh:29-60``) pairs neighbouring elements (2i, 2i+1), so a
+    lane holds both halves of every pair it rotates.  Here the partner of a lane's 16-byte vector
+    lies head_dim/2 elements further on (or back), in the vector of a lane ``head_dim/2 /
+    vec_size`` lanes away in the same wave: the op is a ``CUSTOM_VECTOR_OP`` that fetches the
+    partner's vector with a lane exchange, the kind of op the reference's ``vector_op`` hook
+    exists for (``sideaware.cu:81-83``).  The arithmetic per pair is the same as the interleaved
+    op's: ``(x1*c - x2*s, x2*c + x1*s)`` in fp32, each product rounded before the add, so the
+    result equals the interleaved op on the permuted head bit for bit.
+
+    in0/out0: the activation, (B, T, heads, head_dim), or (B, heads, T, head_dim) with
+    ``heads_first``; in1: the same fp32 table as :func:`rope_header` takes, (T, head_dim/2, 2) of
+    (cos, sin).  With ``heads_at_launch`` the head count is read from ``sideband_value``.
+    head_dim/2 must be a power-of-two number of 16-byte vectors (bf16 / fp16: head_dim = 16, 32,
+    64, 128, 256, 512; fp32: 8 ... 256), so that a head never straddles a 64-lane wave.
+    """
+    if dtype not in _ROPE_HALF_TYPES:
+        raise ValueError("dtype must be 'fp32', 'bf16' or 'fp16'")
+    elem, vec = _ROPE_HALF_TYPES[dtype]
+    half = head_dim // 2
+    lanes = half // vec                                  # lanes between a vector and its partner
+    if head_dim % 2 or half % vec or lanes < 1 or lanes > 32 or lanes & (lanes - 1):
+        raise ValueError("head_dim/2 must be a power-of-two multiple (1..32) of %d elements for %s" % (vec, dtype))
+    if heads_at_launch and heads_first:
+        raise ValueError("with heads_first the head count is not needed: leave heads_at_launch off")
+    name = "sideaware_rope_half_%s_%s_%s_t%d_h%s_d%d" % (
+        "bwd" if backward else "fwd", dtype, "bhtd" if heads_first else "bthd", T,
+        "N" if heads_at_launch else str(n_heads), head_dim)
+    if heads_first:
+        token = "(int)(row % rope_T)"
+    elif heads_at_launch:
+        token = "(int)((row / (size_type)val) % rope_T)"
+    else:
+        token = "(int)((row / rope_heads) % rope_T)"
+    # forward: first half x1*c - x2*s, second half x2*c + x1*s; backward: the signs swap
+    keep_sign, send_sign = ("-", "+") if backward else ("+", "-")
+    lines = ["#define KERNEL_NAME %s\n" % name,
+             # the table is read as plain floats: a lane loads vec_size of them, the (cos, sin) of
+             # the vec_size/2 pairs it rotates
+             "typedef %s o0;\ntypedef %s i0;\ntypedef float i1;\n" % (elem, elem),
+             _UNUSED + "typedef unused o1, o2, o3, i2, i3;\n"]
+    if unrolled is not None:
+        lines.append("#define UNROLLED %d\n" % unrolled)
+    lines.append("constexpr bool reverse_order = false;\n" + _evict([evict_input, False]))
+    lines.append(
+        "constexpr int rope_T = %d;\n"
+        "constexpr int rope_dim = %d;           // elements per head\n"
+        "constexpr int rope_half = %d;          // pairs per head\n"
+        "constexpr int rope_heads = %d;         // heads per token\n"
+        "constexpr int rope_partner_lanes = %d; // lanes between the two halves of a pair\n"
+        "constexpr int rope_vec = %d;           // elements per 16-byte vector\n"
+        % (T, head_dim, half, max(n_heads, 1), lanes, vec))
+    lines.append(
+        "__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,\n"
+        "                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,\n"
+        "                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}\n"
+        "// A lane holds rope_vec elements of one half of a head; the lane rope_partner_lanes away holds\n"
+        "// the same positions of the other half.  The two split the work by position, not by half: the\n"
+        "// lane of the first half rotates the first rope_vec/2 pairs, its partner the rest, so each\n"
+        "// needs only the table entries of its own pairs.  They trade the elements the other needs\n"
+        "// before the rotation and the results the other stores after it: four 32-bit lane exchanges\n"
+        "// per 16-byte vector in all.\n"
+        "// One 32-bit word of the partner lane.  Distances of 1, 2 and 8 lanes are data-parallel\n"
+        "// moves inside a row of 16 lanes, 16 and 32 lanes are gfx950's row and half-wave swaps: all\n"
+        "// run in the vector ALU.  4 lanes goes through the LDS crossbar.  `upper` says whether this\n"
+        "// lane is the one with the higher number of the two.\n"
+        "__device__ __forceinline__ int rope_partner_word(int v, bool upper) {\n"
+        "    if constexpr (rope_partner_lanes == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false);      // quad_perm:[1,0,3,2]\n"
+        "    else if constexpr (rope_partner_lanes == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false); // quad_perm:[2,3,0,1]\n"
+        "    else if constexpr (rope_partner_lanes == 8) return __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false); // row_ror:8\n"
+        "    else if constexpr (rope_partner_lanes == 16) {\n"
+        "        const auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);\n"
+        "        return (int)(upper ? r[0] : r[1]);\n"
+        "    } else if constexpr (rope_partner_lanes == 32) {\n"
+        "        const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);\n"
+        "        return (int)(upper ? r[0] : r[1]);\n"
+        "    } else return __shfl_xor(v, rope_partner_lanes);\n"
+        "}\n"
+        "#define CUSTOM_IDX_FUNC\n"
+        "__device__ __forceinline__ bool indexing(size_type vec_idx, int vec_size,\n"
+        "                         size_type &idx_i0, size_type &idx_i1,\n"
+        "                         size_type &idx_i2, size_type &idx_i3, int* mem, int val) {\n"
+        "    const size_type elem = vec_idx * vec_size;\n"
+        "    const size_type row = elem / rope_dim;                 // (batch, token, head) or (batch, head, token)\n"
+        "    const int token = %s;\n"
+        "    const int in_head = (int)(elem %% rope_dim);\n"
+        "    const bool second = in_head >= rope_half;\n"
+        "    const int pair = (second ? in_head - rope_half + rope_vec / 2 : in_head);   // first pair this lane rotates\n"
+        "    idx_i0 = vec_idx;\n"
+        "    idx_i1 = (size_type)((token * rope_half + pair) / (rope_vec / 2));       // in units of rope_vec floats\n"
+        "    idx_i2 = 0;\n"
+        "    idx_i3 = 0;\n"
+        "    return false;\n"
+        "}\n"
+        "#define CUSTOM_VECTOR_OP\n"
+        "__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size,\n"
+        "                          o0 *out0, o1 *out1, o2 *out2, o3 *out3,\n"
+        "                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,\n"
+        "                          int* sideband_memory, int sideband_value) {\n"
+        "    constexpr int H = rope_vec / 2;                        // pairs per lane\n"
+        "    constexpr int W = H * (int)sizeof(i0) / 4;             // 32-bit words in half a vector\n"
+        "    const bool second = (int)((vec_idx * vec_size) %% rope_dim) >= rope_half;\n"
+        "    // The lane of the first half keeps its lower H elements and gives away the upper H; the lane\n"
+        "    // of the second half the other way round.\n"
+        "    int words[2 * W], mine_w[W], offer[W], got[W];\n"
+        "    __builtin_memcpy(words, in0, 8 * W);\n"
+        "    #pragma unroll\n"
+        "    for (int w = 0; w < W; w++) {\n"
+        "        mine_w[w] = second ? words[W + w] : words[w];\n"
+        "        offer[w] = second ? words[w] : words[W + w];\n"
+        "    }\n"
+        "    #pragma unroll\n"
+        "    for (int w = 0; w < W; w++) got[w] = rope_partner_word(offer[w], second);\n"
+        "    i0 mine[H], theirs[H], keep[H], send[H];\n"
+        "    __builtin_memcpy(mine, mine_w, 4 * W);\n"
+        "    __builtin_memcpy(theirs, got, 4 * W);\n"
+        "    // With m this lane's element of a pair and t the partner's, the first-half lane keeps\n"
+        "    // y1 = m*c - t*s and sends y2 = t*c + m*s; the second-half lane keeps y2 = m*c + t*s and\n"
+        "    // sends y1 = t*c - m*s (backward: the signs swap).  One expression serves both: the sign of\n"
+        "    // the s-products is flipped in the first-half lane, which is exact.\n"
+        "    const unsigned flip = second ? 0u : 0x80000000u;\n"
+        "    #pragma unroll\n"
+        "    for (int i = 0; i < H; i++) {\n"
+        "        const float m = (float)mine[i], t = (float)theirs[i];\n"
+        "        const float c = in1[2 * i], s = in1[2 * i + 1];\n"
+        "        const float ts = __uint_as_float(__float_as_uint(t * s) ^ flip);\n"
+        "        const float ms = __uint_as_float(__float_as_uint(m * s) ^ flip);\n"
+        "        keep[i] = (o0)(m * c %s ts);\n"
+        "        send[i] = (o0)(t * c %s ms);\n"
+        "    }\n"
+        "    __builtin_memcpy(offer, send, 4 * W);\n"
+        "    #pragma unroll\n"
+        "    for (int w = 0; w < W; w++) got[w] = rope_partner_word(offer[w], second);\n"
+        "    __builtin_memcpy(mine_w, keep, 4 * W);\n"
+        "    #pragma unroll\n"
+        "    for (int w = 0; w < W; w++) {\n"
+        "        words[w] = second ? got[w] : mine_w[w];\n"
+        "        words[W + w] = second ? mine_w[w] : got[w];\n"
+        "    }\n"
+        "    __builtin_memcpy(out0, words, 8 * W);\n"
+        "}\n" % (token, keep_sign, send_sign))
+    return "".join(lines).encode()
+
+
 def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = True) -> bytes:
     """bf16 ``y = x*scale + bias``; scale and bias are two fp32 values read from the sideband
     pointer at launch, so one compiled kernel serves every (scale, bias)."""

@@ -145,6 +145,59 @@ def rope_backward_heads_many(tensors, freqs):
     return _rope_heads_many(list(tensors), freqs, True)
 
 
+_ROPE_DTYPES = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
+
+
+def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], heads_first: bool,
+               backward: bool) -> torch.Tensor:
+    assert x.dim() == 4 and x.is_contiguous(), "activations are contiguous (B, T, heads, head_dim) or (B, heads, T, head_dim)"
+    if heads_first:
+        _, heads, T, head_dim = x.shape
+    else:
+        _, T, heads, head_dim = x.shape
+    dtype = _ROPE_DTYPES.get(x.dtype)
+    if dtype is None:
+        raise TypeError("RoPE storage is float32, bfloat16 or float16")
+    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    if out is None:
+        out = x
+    assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
+    key = ("rope_half", T, heads, head_dim, dtype, heads_first, backward)
+    kid = _kernel(key, lambda: headers.rope_half_header(T, heads, head_dim, dtype, backward, heads_first))
+    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+    return out
+
+
+def rope_half_forward(x, freqs, out=None, heads_first: bool = False):
+    """RoPE for the half-split pair layout (element i of a head pairs with element
+    i + head_dim/2, the "rotate_half" convention): (B, T, heads, head_dim), or
+    (B, heads, T, head_dim) with ``heads_first``.  ``freqs`` is the same (T, head_dim) table the
+    interleaved ops take ([t, 2i] = cos, [t, 2i+1] = sin of pair i).  In place unless ``out`` is given."""
+    return _rope_half(x, freqs, out, heads_first, False)
+
+
+def rope_half_backward(dout, freqs, out=None, heads_first: bool = False):
+    return _rope_half(dout, freqs, out, heads_first, True)
+
+
+def rope_half_forward_many(tensors, freqs, backward: bool = False):
+    """Half-split RoPE of several (B, T, heads, head_dim) tensors in place in ONE launch (q and k
+    of a grouped-query model)."""
+    tensors = list(tensors)
+    first = tensors[0]
+    T, head_dim = first.shape[1], first.shape[3]
+    dtype = _ROPE_DTYPES.get(first.dtype)
+    if dtype is None:
+        raise TypeError("RoPE storage is float32, bfloat16 or float16")
+    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    for t in tensors:
+        assert t.dim() == 4 and t.is_contiguous() and t.shape[1] == T and t.shape[3] == head_dim and t.dtype == first.dtype
+    key = ("rope_half_heads_at_launch", T, head_dim, dtype, backward)
+    kid = _kernel(key, lambda: headers.rope_half_header(T, 0, head_dim, dtype, backward, heads_at_launch=True))
+    elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], None, t.shape[2]) for t in tensors])
+    return tensors
+
+
 def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[torch.Tensor] = None):
     """bf16 ``y = x*scale + bias`` in fp32, rounded to nearest even.  ``scale_bias`` is a device
     tensor of two fp32 values, read by the kernel, so changing them costs no compile."""

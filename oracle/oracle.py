@@ -212,3 +212,40 @@ def bf16_ulp_distance(a_bits, b_bits) -> np.ndarray:
         x = x.astype(np.int32)
         return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
     return np.abs(line(_u16(a_bits)) - line(_u16(b_bits)))
+
+
+# ----------------------------------------------------------------------------------------------
+# Half-split pair layout ("rotate_half": element i of a head pairs with element i + HS/2).  The
+# reference has only the interleaved layout (kernel_rope.cuh:29-60, example_llmc_rope.cu:54-86);
+# the half-split op is the same rotation applied to a permuted head, so it is stated here as
+# exactly that: permute, run the restated reference loop, permute back.  tests/test_oracle.py pins
+# it against the formula written out directly (x1*c - x2*s, x2*c + x1*s) in numpy float32, bit for
+# bit, and against a float64 complex product.
+
+def _half_to_interleaved(x: np.ndarray) -> np.ndarray:
+    h = x.shape[-1] // 2
+    return np.ascontiguousarray(np.stack([x[..., :h], x[..., h:]], axis=-1).reshape(x.shape))
+
+
+def _interleaved_to_half(y: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(np.concatenate([y[..., 0::2], y[..., 1::2]], axis=-1))
+
+
+def _bthd(x: np.ndarray, heads_first: bool) -> np.ndarray:
+    return np.ascontiguousarray(np.swapaxes(x, 1, 2)) if heads_first else x
+
+
+def rope_half_forward_heads_f32(inp, freqs, heads_first: bool = False) -> np.ndarray:
+    """inp (B, T, NH, HS) fp32, or (B, NH, T, HS) with heads_first; freqs as for the interleaved op."""
+    y = rope_forward_heads_f32(_half_to_interleaved(_bthd(_f32(inp), heads_first)), freqs)
+    return _bthd(_interleaved_to_half(y), heads_first)
+
+
+def rope_half_backward_heads_f32(dout, freqs, heads_first: bool = False) -> np.ndarray:
+    y = rope_backward_heads_f32(_half_to_interleaved(_bthd(_f32(dout), heads_first)), freqs)
+    return _bthd(_interleaved_to_half(y), heads_first)
+
+
+def rope_half_forward_heads_bf16(inp_bits, freqs, heads_first: bool = False) -> np.ndarray:
+    y = rope_forward_heads_bf16(_half_to_interleaved(_bthd(_u16(inp_bits), heads_first)), freqs)
+    return _bthd(_interleaved_to_half(y), heads_first)

@@ -382,3 +382,16 @@ def test_every_wide_store_is_followed_by_two_wait_states(lib, tmp_path):
                 seen += 1
                 assert lines[i + 1].startswith("s_nop 1"), (variant, lines[i:i + 3])
     assert seen >= 16
+
+
+def test_half_split_rope_headers_compile_and_refuse_heads_that_would_straddle_a_wave(lib):
+    for kw in (dict(dtype="bf16"), dict(dtype="fp32", backward=True), dict(dtype="fp16", heads_first=True),
+               dict(dtype="bf16", heads_at_launch=True)):
+        for variant in (0, 2, 4):
+            rc, log = compile_ok(lib, headers.rope_half_header(4096, 32, 128, **kw), variant)
+            assert rc == 0, (kw, variant, log)
+    rc, log = compile_ok(lib, headers.rope_half_header(64, 2, 8, "fp32"), 0)      # one vector per half
+    assert rc == 0, log
+    for bad in ((96, "bf16"), (24, "fp32"), (1024, "fp32"), (7, "fp32")):           # 6 lanes, 3 lanes, 128 lanes, odd
+        with pytest.raises(ValueError):
+            headers.rope_half_header(16, 2, bad[0], bad[1])

@@ -1,0 +1,106 @@
+"""GPU parity of the half-split ("rotate_half") RoPE op against the CPU oracle, bit for bit.
+
+The op exchanges 16-byte vectors between lanes of a wave, so the cases cover every lane distance
+(1 ... 32 lanes between the halves of a pair), all three storage types, both tensor layouts,
+backward, arrays that end in a partial tile, out of place, several tensors in one launch, and the
+Llama-3-8B q and k at full size.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    t = t.detach().contiguous().cpu()
+    view = {2: torch.int16, 4: torch.int32}[t.element_size()]
+    return t.view(view).numpy().view({2: np.uint16, 4: np.uint32}[t.element_size()])
+
+
+def assert_no_library_error(sa):
+    assert sa.sideaware_last_error() == "", sa.sideaware_last_error()
+
+
+@pytest.mark.parametrize("B,T,H,D", [(1, 8, 1, 8), (2, 33, 3, 16), (1, 64, 5, 32), (2, 40, 7, 64), (1, 130, 3, 128),
+                                     (2, 16, 2, 256)])
+def test_fp32_forward_and_backward_vs_oracle(sa, B, T, H, D):
+    from l2_torch_alloc_amd import ops
+    g = torch.Generator().manual_seed(B * 1000 + T + D)
+    x = torch.randn(B, T, H, D, generator=g)
+    table = O.freqs_cis(D, T, 10000.0)
+    freqs = torch.from_numpy(table).cuda()
+    y = ops.rope_half_forward(x.cuda(), freqs)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    want = O.rope_half_forward_heads_f32(x.numpy(), table)
+    assert np.array_equal(bits(y), want.view(np.uint32))
+    # backward, out of place, from the forward result
+    dx = torch.empty_like(y)
+    ops.rope_half_backward(y, freqs, out=dx)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(dx), O.rope_half_backward_heads_f32(want, table).view(np.uint32))
+    assert np.array_equal(bits(y), want.view(np.uint32))             # the input of an out-of-place launch is untouched
+
+
+@pytest.mark.parametrize("B,T,H,D", [(1, 8, 2, 16), (2, 33, 3, 32), (3, 40, 5, 64), (2, 100, 9, 128), (1, 24, 2, 512)])
+def test_bf16_vs_oracle_both_layouts(sa, B, T, H, D):
+    from l2_torch_alloc_amd import ops
+    g = torch.Generator().manual_seed(7 * T + D)
+    x = torch.randn(B, T, H, D, generator=g).to(torch.bfloat16)
+    table = O.freqs_cis(D, T, 500000.0)
+    freqs = torch.from_numpy(table).cuda()
+    want = O.rope_half_forward_heads_bf16(bits(x), table)
+    y = ops.rope_half_forward(x.cuda(), freqs)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(y), want)
+    # (B, heads, T, D): the same numbers, transposed
+    xt = x.transpose(1, 2).contiguous()
+    yt = ops.rope_half_forward(xt.cuda(), freqs, heads_first=True)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(yt), np.ascontiguousarray(np.swapaxes(want, 1, 2)))
+    assert np.array_equal(bits(yt), O.rope_half_forward_heads_bf16(bits(xt), table, heads_first=True))
+
+
+def test_fp16_vs_the_oracles_fp32_result_narrowed_by_numpy(sa):
+    from l2_torch_alloc_amd import ops
+    B, T, H, D = 2, 50, 3, 64
+    x = torch.randn(B, T, H, D, generator=torch.Generator().manual_seed(5)).to(torch.float16)
+    table = O.freqs_cis(D, T, 10000.0)
+    y = ops.rope_half_forward(x.cuda(), torch.from_numpy(table).cuda())
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    want = O.rope_half_forward_heads_f32(x.float().numpy(), table).astype(np.float16)
+    assert np.array_equal(bits(y), want.view(np.uint16))
+
+
+def test_q_and_k_in_one_launch_at_llama3_size_vs_oracle(sa):
+    from l2_torch_alloc_amd import ops
+    B, T, D = 8, 4096, 128
+    table = O.freqs_cis(D, T, 500000.0)
+    freqs = torch.from_numpy(table).cuda()
+    g = torch.Generator().manual_seed(12)
+    q_h = torch.randn(B, T, 32, D, generator=g).to(torch.bfloat16)
+    k_h = torch.randn(B, T, 8, D, generator=g).to(torch.bfloat16)
+    q, k = q_h.cuda(), k_h.cuda()
+    ops.rope_half_forward_many([q, k], freqs)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(k), O.rope_half_forward_heads_bf16(bits(k_h), table))
+    # q: the first and the last batch entries against the oracle, all of it against the one-tensor launch
+    want0 = O.rope_half_forward_heads_bf16(bits(q_h[:1]), table)
+    want7 = O.rope_half_forward_heads_bf16(bits(q_h[7:]), table)
+    got = bits(q)
+    assert np.array_equal(got[:1], want0) and np.array_equal(got[7:], want7)
+    q2 = ops.rope_half_forward(q_h.cuda(), freqs)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(q2), got)
+    # backward of both in one launch brings the inputs back to within rounding
+    ops.rope_half_forward_many([q, k], freqs, backward=True)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert float((q.float().cpu() - q_h.float()).abs().max()) <= 0.0625

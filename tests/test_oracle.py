@@ -294,3 +294,51 @@ def test_fp16_narrowing_used_for_fp16_rope_is_ieee_round_to_nearest_even():
     mid = (a + b) / 2                                                  # exact in float32
     got = mid.astype(np.float16).view(np.uint16)
     assert np.array_equal(got, np.where(lo % 2 == 0, lo, lo + 1))
+
+
+# ---------------------------------------------------------------- half-split pair layout
+
+def _direct_half_rope(x, f, backward=False):
+    """(x1*c - x2*s, x2*c + x1*s) written out in numpy float32: every product and sum rounded on
+    its own, in the order the interleaved formula has them (example_llmc_rope.cu:70-81)."""
+    h = x.shape[-1] // 2
+    c = f[:, 0::2][None, :, None, :].astype(np.float32)
+    s = f[:, 1::2][None, :, None, :].astype(np.float32)
+    x1, x2 = x[..., :h], x[..., h:]
+    if backward:
+        return np.concatenate([x1 * c + x2 * s, x2 * c - x1 * s], axis=-1)
+    return np.concatenate([x1 * c - x2 * s, x2 * c + x1 * s], axis=-1)
+
+
+@pytest.mark.parametrize("B,T,NH,HS", [(2, 7, 3, 8), (1, 16, 8, 64), (2, 5, 4, 128)])
+def test_rope_half_split_layout_vs_the_formula_written_out(B, T, NH, HS):
+    x = rng(B * T + HS).standard_normal((B, T, NH, HS)).astype(np.float32)
+    f = O.freqs_cis(HS, T, 10000.0)
+    y = O.rope_half_forward_heads_f32(x, f)
+    assert np.array_equal(y.view(np.uint32), _direct_half_rope(x, f).view(np.uint32))
+    # a float64 complex product of (x1 + i x2) with (cos + i sin)
+    z = (x[..., :HS // 2].astype(np.float64) + 1j * x[..., HS // 2:]) * \
+        (f[:, 0::2].astype(np.float64) + 1j * f[:, 1::2])[None, :, None, :]
+    np.testing.assert_allclose(y[..., :HS // 2], z.real, atol=1e-6, rtol=1e-6)
+    np.testing.assert_allclose(y[..., HS // 2:], z.imag, atol=1e-6, rtol=1e-6)
+    # token 0 is the identity; a dropped permutation would show as the interleaved result
+    assert np.array_equal(y[:, 0].view(np.uint32), x[:, 0].view(np.uint32))
+    if T > 1 and HS > 2:
+        assert not np.array_equal(y, O.rope_forward_heads_f32(x, f))
+    # backward: the formula written out, and the inverse of forward
+    dx = O.rope_half_backward_heads_f32(y, f)
+    assert np.array_equal(dx.view(np.uint32), _direct_half_rope(y, f, backward=True).view(np.uint32))
+    np.testing.assert_allclose(dx, x, atol=2e-6, rtol=2e-6)
+    # (B, heads, T, HS) is the same op on the transposed tensor
+    xt = np.ascontiguousarray(np.swapaxes(x, 1, 2))
+    assert np.array_equal(O.rope_half_forward_heads_f32(xt, f, heads_first=True), np.swapaxes(y, 1, 2))
+
+
+def test_rope_half_split_bf16_vs_torch_rounding():
+    B, T, NH, HS = 2, 6, 3, 32
+    xb = O.f32_to_bf16(rng(9).standard_normal((B, T, NH, HS)).astype(np.float32))
+    f = O.freqs_cis(HS, T, 500000.0)
+    got = O.rope_half_forward_heads_bf16(xb, f)
+    xw = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).to(torch.float32).numpy()
+    want = torch.from_numpy(_direct_half_rope(xw, f)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
