@@ -373,24 +373,27 @@ def mxfp8_quantize_header(unrolled: int | None = None) -> bytes:
         "    #pragma unroll\n"
         "    for (int i = 0; i < 8; i++) { v[i] = (float)in0[i]; amax = fmaxf(amax, fabsf(v[i])); }\n"
         "    // a block of 32 elements is 4 neighbouring lanes: lanes 4k..4k+3 of the wave\n"
-        "    amax = fmaxf(amax, __shfl_xor(amax, 1));\n"
-        "    amax = fmaxf(amax, __shfl_xor(amax, 2));\n"
+        "    // (data-parallel moves inside each group of four lanes: quad_perm [1,0,3,2], then [2,3,0,1])\n"
+        "    amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0xB1, 0xf, 0xf, false)));\n"
+        "    amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0x4E, 0xf, 0xf, false)));\n"
         "    // floor(log2(amax)) is the exponent field of the float (a bf16 subnormal widens to an\n"
         "    // fp32 subnormal with field 0, far below the clamp anyway)\n"
         "    int shared_exp = (int)((__float_as_uint(amax) >> 23) & 0xff) - 127 - 8;\n"
         "    if (amax == 0.0f || shared_exp < -127) shared_exp = -127;\n"
         "    if (shared_exp > 127) shared_exp = 127;\n"
         "    if ((vec_idx & 3) == 0) ((unsigned char*)sideband_memory)[vec_idx >> 2] = (unsigned char)(shared_exp + 127);\n"
+        "    // two conversions fill one 32-bit word with four E4M3 bytes: the second writes the upper half\n"
+        "    int words[2] = {0, 0};\n"
         "    #pragma unroll\n"
         "    for (int i = 0; i < 8; i += 2) {\n"
-        "        // two exact power-of-two steps: 2^127 and 2^-127 are not both normal floats\n"
+        "        // ldexpf scales exactly over the whole range (2^127 and 2^-127 are not both normal floats)\n"
         "        float a = ldexpf(v[i], -shared_exp), b = ldexpf(v[i + 1], -shared_exp);\n"
-        "        a = fminf(fmaxf(a, -448.0f), 448.0f);\n"
-        "        b = fminf(fmaxf(b, -448.0f), 448.0f);\n"
-        "        const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);\n"
-        "        out0[i] = (unsigned char)(packed & 0xff);\n"
-        "        out0[i + 1] = (unsigned char)((packed >> 8) & 0xff);\n"
+        "        a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);\n"
+        "        b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);\n"
+        "        words[i / 4] = (i & 2) ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, words[i / 4], true)\n"
+        "                               : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, words[i / 4], false);\n"
         "    }\n"
+        "    __builtin_memcpy(out0, words, 8);\n"
         "}\n")
     return "".join(lines).encode()
 
