@@ -279,6 +279,13 @@ def ceiling(steps, nbytes=GiB, pairs=2, only=None):
         for wait in (0, WAIT_STORES):
             run("copy persistent bursts k=%d block=%d grid=%d%s nt" % (k, block, grid, " wait-stores" if wait else ""),
                 2 * nbytes, persistent(k, block, grid, hints["nt"] | wait, 0))
+    # persistent grids again, software-pipelined: the next chunk's loads are issued before the
+    # current chunk's stores (flag 16), beside the same grid without
+    for k, block, grid in ((1, 256, 1024), (1, 256, 2048), (2, 256, 1024), (2, 256, 2048), (4, 256, 1024),
+                           (1, 256, 4096), (2, 256, 4096), (1, 1024, 512), (2, 1024, 256)):
+        for prefetch in (0, 16):
+            run("copy persistent%s k=%d block=%d grid=%d nt" % (" prefetch" if prefetch else " no-prefetch", k, block, grid),
+                2 * nbytes, persistent(k, block, grid, hints["nt"] | prefetch, 0))
     # the workgroup -> address map: stripes of 2^r tiles per XCD, from tile-by-tile round robin (r = 0:
     # consecutive workgroups take consecutive 4 KiB chunks) to 2 MiB runs per XCD
     for r in range(0, 10):

@@ -17,6 +17,7 @@ enum : int {
     kNtStores = 2,         // stores carry the nontemporal hint
     kLaneContiguous = 4,   // a lane takes K consecutive vectors instead of K vectors a block apart
     kWaitStores = 8,       // persistent kernels: stores are acknowledged before the next loads are issued
+    kPrefetch = 16,        // persistent copies: the next chunk's loads are issued before this chunk's stores
     kSplitRoles = 16,      // tile kernel: workgroup pairs alternate between reading src and filling dst
 };
 
@@ -290,6 +291,35 @@ __global__ __launch_bounds__(1024) void persistent_kernel(v4i* dst, const v4i* s
     }
 }
 
+// The same fixed grid for a copy, software-pipelined: the loads of a workgroup's next chunk are in
+// flight while the current chunk is stored, so a workgroup always has reads and writes outstanding
+// instead of alternating between them.
+template <int K, bool NTL, bool NTS>
+__global__ __launch_bounds__(1024) void persistent_prefetch_kernel(v4i* dst, const v4i* src, long long n_chunks, int flags,
+                                                                   unsigned period_ticks, int* sink) {
+    const unsigned B = blockDim.x, tid = threadIdx.x;
+    const long long chunk = (long long)B * K;
+    long long c = blockIdx.x;
+    if (c >= n_chunks) return;
+    v4i cur[K], nxt[K];
+    #pragma unroll
+    for (int k = 0; k < K; k++) cur[k] = ld<NTL>(src + c * chunk + tid + (long long)k * B);
+    for (;;) {
+        const long long cn = c + gridDim.x;
+        const bool more = cn < n_chunks;                       // uniform across the workgroup
+        if (more) {
+            #pragma unroll
+            for (int k = 0; k < K; k++) nxt[k] = ld<NTL>(src + cn * chunk + tid + (long long)k * B);
+        }
+        #pragma unroll
+        for (int k = 0; k < K; k++) st<NTS>(dst + c * chunk + tid + (long long)k * B, cur[k]);
+        if (!more) break;
+        #pragma unroll
+        for (int k = 0; k < K; k++) cur[k] = nxt[k];
+        c = cn;
+    }
+}
+
 typedef void (*tile_fn)(v4i*, const v4i*, unsigned, int, int*, unsigned long long*);
 typedef void (*persistent_fn)(v4i*, const v4i*, long long, int, unsigned, int*);
 
@@ -306,6 +336,14 @@ static tile_fn pick_tile(int flags) {
 
 template <int K>
 static persistent_fn pick_persistent(int flags) {
+    if (flags & kPrefetch) {
+        switch (flags & 3) {
+            case 0: return persistent_prefetch_kernel<K, false, false>;
+            case 1: return persistent_prefetch_kernel<K, true, false>;
+            case 2: return persistent_prefetch_kernel<K, false, true>;
+            default: return persistent_prefetch_kernel<K, true, true>;
+        }
+    }
     switch (flags & 3) {
         case 0: return persistent_kernel<K, false, false>;
         case 1: return persistent_kernel<K, true, false>;
@@ -409,6 +447,8 @@ int hbm_ceiling_persistent(void* dst, const void* src, size_t bytes, int k, int 
     if (block < 64 || block > 1024 || (block & (block - 1))) return fail("block must be a power of two in 64..1024");
     if (grid < 1 || grid > (1 << 20)) return fail("grid out of range");
     if (!dst && !src) return fail("nothing to do");
+    if ((flags & kPrefetch) && (!dst || !src || period_ticks)) return fail("prefetch is for plain copies");
+    if ((flags & kPrefetch) && k > 8) return fail("prefetch: k at most 8");
     if (!sink) return fail("sink must point at four bytes of device memory");
     const size_t chunk_bytes = (size_t)k * block * 16;
     if (bytes == 0 || bytes % chunk_bytes) return fail("bytes must be a whole number of chunks");
