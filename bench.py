@@ -656,7 +656,7 @@ def main():
     if not args.quick:
         warm = bench_copy(256 * MiB, args.steps, args.warmup, "uint8", seed=0)
         warm["note"] = ("cache-assisted: the same (src, dst) pair copied back to back, so the destination, exactly the "
-                        "size of the Infinity Cache and stored plainly, is partly still cached from the launch before")
+                        "size of the Infinity Cache and left cacheable, is partly still cached from the launch before")
         log("copy 256 MiB, one pair in a loop:", warm)
         also["copy_256MiB_one_pair_in_a_loop"] = warm
     if args.quick:

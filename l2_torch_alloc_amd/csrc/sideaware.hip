@@ -35,7 +35,7 @@ static const char* kKernelTemplate =
 
 // Kernel id 0: a bit-exact copy, four bytes per element so that sixteen bytes make one vector.
 // The source is marked evict (read once, with the streaming hint) and UNROLLED is left at 1: one
-// workgroup moves one 4 KiB chunk.  The destination is written plainly while it fits the Infinity
+// workgroup moves one 4 KiB chunk.  The destination is left cacheable while it fits the Infinity
 // Cache, so the next kernel finds it there, and with the streaming hint beyond that.
 static const char* kMemcpyHeader = R"SA_HDR(
 #define KERNEL_NAME sideaware_copy
@@ -603,7 +603,7 @@ static_assert(sizeof(SegmentArgs) == 128 && sizeof(BatchArgs) == 128 * kMaxSegme
               "the device side declares the same layout");
 
 // The instantiation a launch over these arrays needs.  Index width: 32-bit below 2 GiB, 64-bit from
-// there on.  Cache class: arrays whose result fits the Infinity Cache (written plainly, so the next
+// there on.  Cache class: arrays whose result fits the Infinity Cache (left cacheable, so the next
 // kernel finds it there) and larger ones (everything streams).  In place (o0 written over i0) is a
 // class of its own below the cache size: see the template's notes on cache policy.  A base that is
 // not 2 MiB-aligned gets the instantiation whose `aligned_2MiB` is false, as in the reference
