@@ -104,3 +104,38 @@ def test_q_and_k_in_one_launch_at_llama3_size_vs_oracle(sa):
     torch.cuda.synchronize()
     assert_no_library_error(sa)
     assert float((q.float().cpu() - q_h.float()).abs().max()) <= 0.0625
+
+
+def test_batched_launches_replay_from_a_hip_graph(sa):
+    # the batched launch carries its segment table in the kernel arguments (no device memory is
+    # written by the call), so it is captured like any kernel: q and k of both pair layouts
+    from l2_torch_alloc_amd import ops
+    T, D = 96, 128
+    table = O.freqs_cis(D, T, 500000.0)
+    freqs = torch.from_numpy(table).cuda()
+    g = torch.Generator().manual_seed(21)
+    q0 = torch.randn(2, T, 8, D, generator=g).to(torch.bfloat16)
+    k0 = torch.randn(2, T, 2, D, generator=g).to(torch.bfloat16)
+    q, k, q2, k2 = q0.cuda(), k0.cuda(), q0.cuda(), k0.cuda()
+    ops.rope_half_forward_many([q.clone(), k.clone()], freqs)          # compiled outside the capture
+    ops.rope_forward_heads_many([q2.clone(), k2.clone()], freqs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.rope_half_forward_many([q, k], freqs)
+            ops.rope_forward_heads_many([q2, k2], freqs)
+    torch.cuda.current_stream().wait_stream(side)
+    want_q, want_k = O.rope_half_forward_heads_bf16(bits(q0), table), O.rope_half_forward_heads_bf16(bits(k0), table)
+    want_q2, want_k2 = O.rope_forward_heads_bf16(bits(q0), table), O.rope_forward_heads_bf16(bits(k0), table)
+    for trial in range(3):
+        for dst, src in ((q, q0), (k, k0), (q2, q0), (k2, k0)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(q), want_q) and np.array_equal(bits(k), want_k), trial
+        assert np.array_equal(bits(q2), want_q2) and np.array_equal(bits(k2), want_k2), trial
+    assert_no_library_error(sa)
