@@ -27,6 +27,17 @@ def _kernel(key: Tuple, make_header) -> int:
     return kid
 
 
+def _elementwise(*args) -> None:
+    """The elementwise op.  Eager code goes straight to the op's implementation, the function
+    ``torch.ops.sideaware.elementwise`` dispatches to, and saves the dispatcher's per-call cost
+    (about a microsecond of a small launch); under ``torch.compile`` the call goes through the
+    registered op, which the tracer keeps as one opaque node."""
+    if torch.compiler.is_compiling():
+        torch.ops.sideaware.elementwise(*args)
+    else:
+        wrapper.sideaware_elementwise(*args)
+
+
 def freqs_cis_table(head_dim: int, end: int, theta: float, use_scaled: bool = False) -> torch.Tensor:
     """(end, head_dim) fp32 table on the host: [t, 2i] = cos(t*f_i), [t, 2i+1] = sin(t*f_i),
     f_i = theta^(-2i/head_dim) in fp32, optionally with the Llama-3.1 wavelength rescaling
@@ -47,6 +58,9 @@ def freqs_cis_table(head_dim: int, end: int, theta: float, use_scaled: bool = Fa
     return table
 
 
+_ROPE_DTYPES = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
+
+
 def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q: int, n_kv: int,
           layout: str, backward: bool) -> torch.Tensor:
     assert x.dim() == 4, "activations are (B, T, heads, head_dim)"
@@ -55,25 +69,23 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
         assert heads == n_q + 2 * n_kv, "packed QKV needs n_q + 2*n_kv heads"
     else:
         n_q, n_kv = heads, 0
-    if x.dtype == torch.float32:
-        dtype = "fp32"
-    elif x.dtype == torch.bfloat16:
-        dtype = "bf16"
-    elif x.dtype == torch.float16:
-        dtype = "fp16"
-    else:
+    dtype = _ROPE_DTYPES.get(x.dtype)
+    if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
-    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    assert freqs.dtype == torch.float32 and freqs.shape == (T, head_dim)
     if out is None:
         out = x
-    assert out.shape == x.shape and out.dtype == x.dtype
-    if layout == "qkv" and out.data_ptr() != x.data_ptr():
-        # value heads are skipped by the kernel (neither read nor written): out of place they
-        # have to be carried over by a copy first
-        torch.ops.sideaware.memcpy(out, x)
-    key = ("rope", T, n_q, n_kv, head_dim, dtype, layout, backward)
-    kid = _kernel(key, lambda: headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout, backward))
-    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+    else:
+        assert out.shape == x.shape and out.dtype == x.dtype
+        if layout == "qkv" and out.data_ptr() != x.data_ptr():
+            # value heads are skipped by the kernel (neither read nor written): out of place they
+            # have to be carried over by a copy first
+            torch.ops.sideaware.memcpy(out, x)
+    key = (T, n_q, n_kv, head_dim, dtype, layout, backward)
+    kid = _kernel_ids.get(key)
+    if kid is None:
+        kid = _kernel(key, lambda: headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout, backward))
+    _elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
     return out
 
 
@@ -115,7 +127,7 @@ def elementwise_batch(kernel_id: int, segments) -> None:
             seg.inp[i] = wrapper._check(t, "in%d" % i) or None
         seg.sideband_memory = sideband.data_ptr() if sideband is not None else None
         seg.sideband_value = int(value)
-    device, stream = torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream
+    device, stream = wrapper._device_and_stream()
     wrapper.library().sideaware_elementwise_batch(kernel_id, len(arr), arr, device, stream)
 
 
@@ -123,7 +135,7 @@ def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool):
     first = tensors[0]
     assert first.dim() == 4, "activations are (B, T, heads, head_dim)"
     T, head_dim = first.shape[1], first.shape[3]
-    dtype = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}.get(first.dtype)
+    dtype = _ROPE_DTYPES.get(first.dtype)
     if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
     assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
@@ -145,9 +157,6 @@ def rope_backward_heads_many(tensors, freqs):
     return _rope_heads_many(list(tensors), freqs, True)
 
 
-_ROPE_DTYPES = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
-
-
 def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], heads_first: bool,
                backward: bool) -> torch.Tensor:
     assert x.dim() == 4 and x.is_contiguous(), "activations are contiguous (B, T, heads, head_dim) or (B, heads, T, head_dim)"
@@ -164,7 +173,7 @@ def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor]
     assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
     key = ("rope_half", T, heads, head_dim, dtype, heads_first, backward)
     kid = _kernel(key, lambda: headers.rope_half_header(T, heads, head_dim, dtype, backward, heads_first))
-    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+    _elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
     return out
 
 
@@ -205,7 +214,7 @@ def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[tor
     if out is None:
         out = torch.empty_like(x)
     kid = _kernel(("scale_bias_bf16",), headers.scale_bias_bf16_header)
-    torch.ops.sideaware.elementwise(kid, out, None, None, None, x, None, None, None, scale_bias, 0, 0, 0)
+    _elementwise(kid, out, None, None, None, x, None, None, None, scale_bias, 0, 0, 0)
     return out
 
 
@@ -219,7 +228,7 @@ def mxfp8_quantize(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Op
         scales = torch.empty(x.numel() // 32, dtype=torch.uint8, device=x.device)
     assert q.dtype == torch.uint8 and q.numel() == x.numel() and scales.numel() == x.numel() // 32
     kid = _kernel(("mxfp8_quantize",), headers.mxfp8_quantize_header)
-    device, stream = torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream
+    device, stream = wrapper._device_and_stream()
     # num_bytes is the byte length of the wider array, the bf16 input, which the custom-op wrapper
     # cannot know (it sizes the launch from out0, as the reference's does): call the C entry point.
     wrapper.library().sideaware_elementwise(kid, x.numel() * 2, q.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
@@ -236,12 +245,12 @@ def mxfp8_dequantize(q: torch.Tensor, scales: torch.Tensor, out: Optional[torch.
     assert out.dtype == torch.bfloat16 and out.numel() == q.numel()
     kid = _kernel(("mxfp8_dequantize",), headers.mxfp8_dequantize_header)
     # out0 is the wider array, so the custom op's own sizing (from out0) is the right one
-    torch.ops.sideaware.elementwise(kid, out, None, None, None, q, None, None, None, scales, 0, 0, 0)
+    _elementwise(kid, out, None, None, None, q, None, None, None, scales, 0, 0, 0)
     return out
 
 
 def fill_int32(out: torch.Tensor, value: int):
     """Writes a 32-bit pattern over ``out`` (byte size a multiple of 16): an output-only op."""
     kid = _kernel(("fill",), headers.fill_header)
-    torch.ops.sideaware.elementwise(kid, out, None, None, None, None, None, None, None, None, int(value), 0, 0)
+    _elementwise(kid, out, None, None, None, None, None, None, None, None, int(value), 0, 0)
     return out

@@ -204,18 +204,28 @@ def _refresh_metadata() -> None:
 # The three ops.  Exposed through torch.ops.sideaware.* so that they trace under torch.compile.
 # ------------------------------------------------------------------------------------------------
 
-def _device_and_stream():
-    return torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream
+# The raw handle of the current stream of a device without building a torch.cuda.Stream object
+# (a third of the cost of a small launch); older PyTorch builds lack the private accessor.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _device_and_stream(t: Optional[torch.Tensor] = None):
+    """(device index, current stream handle): of the device the given tensor lives on, or of the
+    current device."""
+    device = t.get_device() if t is not None else torch.cuda.current_device()
+    if _raw_stream is not None:
+        return device, _raw_stream(device)
+    return device, torch.cuda.current_stream(device).cuda_stream
 
 
 def _check(t: Optional[torch.Tensor], name: str) -> int:
     """Address of a contiguous, 16-byte aligned device tensor; 0 for None."""
     if t is None:
         return 0
-    assert t.device.type == "cuda", name + " must be on the GPU"
+    assert t.is_cuda, name + " must be on the GPU"
     assert t.is_contiguous(), name + " must be contiguous"
     ptr = t.data_ptr()
-    assert ptr % 16 == 0, name + " must be 16-byte aligned"
+    assert not ptr & 15, name + " must be 16-byte aligned"
     return ptr
 
 
@@ -223,8 +233,8 @@ def sideaware_memcpy(dst: torch.Tensor, src: torch.Tensor) -> None:
     assert dst.dtype == src.dtype, "Source and destination must have the same dtype"
     assert dst.numel() >= src.numel(), "Destination tensor must be at least as large as source"
     dst_ptr, src_ptr = _check(dst, "dst"), _check(src, "src")
-    device, stream = _device_and_stream()
-    library().sideaware_memcpy(dst_ptr, src_ptr, src.numel() * src.element_size(), device, stream)
+    device, stream = _device_and_stream(dst)
+    (_lib or library()).sideaware_memcpy(dst_ptr, src_ptr, src.numel() * src.element_size(), device, stream)
 
 
 def sideaware_one_to_one(kernel_id: int, dst: torch.Tensor, src: Optional[torch.Tensor]) -> None:
@@ -232,8 +242,8 @@ def sideaware_one_to_one(kernel_id: int, dst: torch.Tensor, src: Optional[torch.
     num_bytes = dst.numel() * dst.element_size() if dst is not None else 0
     assert num_bytes > 0
     dst_ptr, src_ptr = _check(dst, "dst"), _check(src, "src")
-    device, stream = _device_and_stream()
-    library().sideaware_one_to_one(kernel_id, num_bytes, dst_ptr, src_ptr, device, stream)
+    device, stream = _device_and_stream(dst)
+    (_lib or library()).sideaware_one_to_one(kernel_id, num_bytes, dst_ptr, src_ptr, device, stream)
 
 
 def sideaware_elementwise(kernel_id: int,
@@ -246,12 +256,13 @@ def sideaware_elementwise(kernel_id: int,
     # The byte count is taken from out0, as the reference does (test.py:114-116).
     num_bytes = out0.numel() * out0.element_size() if out0 is not None else 0
     assert num_bytes > 0
-    outs = [_check(t, "out%d" % i) for i, t in enumerate((out0, out1, out2, out3))]
-    ins = [_check(t, "in%d" % i) for i, t in enumerate((in0, in1, in2, in3))]
-    sideband_ptr = sideband_tensor.data_ptr() if sideband_tensor is not None else 0
-    device, stream = _device_and_stream()
-    library().sideaware_elementwise(kernel_id, num_bytes, *outs, *ins, sideband_ptr, sideband_value,
-                                    parallel_chunks, forced_sm_per_side, device, stream)
+    device, stream = _device_and_stream(out0)
+    (_lib or library()).sideaware_elementwise(
+        kernel_id, num_bytes,
+        _check(out0, "out0"), _check(out1, "out1"), _check(out2, "out2"), _check(out3, "out3"),
+        _check(in0, "in0"), _check(in1, "in1"), _check(in2, "in2"), _check(in3, "in3"),
+        sideband_tensor.data_ptr() if sideband_tensor is not None else 0, sideband_value,
+        parallel_chunks, forced_sm_per_side, device, stream)
 
 
 _op_library = None

@@ -273,3 +273,23 @@ def test_multi_stream_churn_keeps_contents(sa):
     assert checked > 1000
     assert after["stream_syncs"] > before["stream_syncs"] + 100      # hand-overs happened, ordered on the device
     assert after["failures"] == before["failures"] and sa.sideaware_last_error() == ""
+
+
+def test_ready_made_ops_under_torch_compile(sa):
+    # eager calls go straight to the op's implementation; while tracing, the same calls go through
+    # torch.ops.sideaware.elementwise, which the tracer keeps as one opaque node
+    from l2_torch_alloc_amd import ops
+    x0 = torch.randn(2, 32, 4, 64, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).cuda()
+    freqs = ops.freqs_cis_table(64, 32, 10000.0).cuda()
+    sb = torch.tensor([1.5, -0.25], dtype=torch.float32, device="cuda")
+    eager = ops.scale_bias_bf16(ops.rope_forward_heads(x0.clone(), freqs), sb)
+
+    @torch.compile(fullgraph=True)
+    def step(x, freqs, sb):
+        y = ops.rope_forward_heads(x, freqs)
+        return ops.scale_bias_bf16(y, sb)
+
+    out = step(x0.clone(), freqs, sb)
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager)
+    assert sa.sideaware_last_error() == ""
