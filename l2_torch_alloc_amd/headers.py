@@ -48,7 +48,7 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
                 layout: str = "qkv", backward: bool = False, unrolled: int | None = 2,
                 reverse_order: bool = False, evict_input: bool = True,
                 stream_input: bool | None = None, stream_output: bool | None = None,
-                heads_at_launch: bool = False) -> bytes:
+                heads_at_launch: bool = False, positions: bool = False) -> bytes:
     """RoPE forward (or backward) in place or out of place.
 
     layout "qkv":   one tensor (B, T, n_q + 2*n_kv, head_dim); q and k heads are rotated, the
@@ -63,6 +63,11 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     ``heads_at_launch`` (layout "heads" only): the number of heads per token is not baked into the
     text but read from the launch's ``sideband_value``, so one compiled kernel serves q and k of a
     grouped-query model and both can go out in one batched launch (``n_q`` is then ignored).
+
+    ``positions`` (layout "heads" only): a token's table row is not its index in the sequence but
+    an int32 read from the launch's sideband pointer, one per token of the flattened (B, T) axes:
+    decoding steps and packed batches of sequences at arbitrary positions (``T`` then only names
+    the kernel).  The table must have a row for every position that occurs.
     """
     if dtype not in _ROPE_TYPES:
         raise ValueError("dtype must be 'fp32', 'bf16' or 'fp16'")
@@ -76,13 +81,14 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
     half = head_dim // 2
     if half % pairs_per_vec:
         raise ValueError("head_dim/2 must be a multiple of %d for %s" % (pairs_per_vec, dtype))
-    if heads_at_launch and layout != "heads":
-        raise ValueError("heads_at_launch needs layout 'heads'")
+    if (heads_at_launch or positions) and layout != "heads":
+        raise ValueError("heads_at_launch and positions need layout 'heads'")
     total_heads = n_q + 2 * n_kv if layout == "qkv" else n_q
     rotated_heads = n_q + n_kv if layout == "qkv" else n_q
     sign_a, sign_b = ("+", "-") if backward else ("-", "+")
 
-    name = "sideaware_rope_%s_%s_%s_t%d_h%s_%d_d%d" % ("bwd" if backward else "fwd", dtype, layout, T,
+    name = "sideaware_rope_%s_%s_%s_t%s_h%s_%d_d%d" % ("bwd" if backward else "fwd", dtype, layout,
+                                                        "pos" if positions else str(T),
                                                         "N" if heads_at_launch else str(n_q),
                                                         n_kv if layout == "qkv" else 0, head_dim)
     lines = ["#define KERNEL_NAME %s\n" % name, decl]
@@ -117,23 +123,25 @@ def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
         "}\n" % (widen % "in0.x", widen % "in0.y", sign_a, sign_b, narrow % "y_re", narrow % "y_im"))
     # A 16-byte vector holds pairs_per_vec consecutive pairs of one head of one token, so one
     # decode serves the whole vector: the table row of the token, at the head-local pair.
-    if heads_at_launch:
+    if heads_at_launch or positions:
         # every head is rotated; the only thing the head count decides is where a token's row ends
+        heads_expr = "(size_type)val" if heads_at_launch else "(size_type)rope_heads"
+        token_expr = "mem[row]" if positions else "(int)(row % rope_T)"
         lines.append(
             "#define CUSTOM_IDX_FUNC\n"
             "__device__ __forceinline__ bool indexing(size_type vec_idx, int vec_size,\n"
             "                         size_type &idx_i0, size_type &idx_i1,\n"
             "                         size_type &idx_i2, size_type &idx_i3, int* mem, int val) {\n"
             "    const size_type pair = vec_idx * vec_size;\n"
-            "    const size_type row = (pair / rope_half) / (size_type)val;      // val: heads per token\n"
-            "    const int token = (int)(row % rope_T);\n"
-            "    const int local = (int)(pair % rope_half);\n"
+            "    const size_type row = (pair / rope_half) / %s;      // the token, counted over batch and sequence\n"
+            "    const int token = %s;\n"
+            "    const int local = (int)(pair %% rope_half);\n"
             "    idx_i0 = vec_idx;\n"
-            "    idx_i1 = (size_type)((token * rope_half + local) / vec_size);\n"
+            "    idx_i1 = (size_type)(((size_type)token * rope_half + local) / vec_size);\n"
             "    idx_i2 = 0;\n"
             "    idx_i3 = 0;\n"
             "    return false;\n"
-            "}\n")
+            "}\n" % (heads_expr, token_expr))
         return "".join(lines).encode()
     lines.append(
         "#define CUSTOM_IDX_FUNC\n"
@@ -163,7 +171,7 @@ _ROPE_HALF_TYPES = {
 
 def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", backward: bool = False,
                      heads_first: bool = False, heads_at_launch: bool = False, unrolled: int | None = 2,
-                     evict_input: bool = True) -> bytes:
+                     evict_input: bool = True, positions: bool = False) -> bytes:
     """RoPE for the half-split pair layout ("rotate_half": element i of a head is paired with
     element i + head_dim/2, as Hugging Face / GPT-NeoX style models store q and k), forward or
     backward, in place or out of place.
@@ -179,7 +187,9 @@ def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", b
 
     in0/out0: the activation, (B, T, heads, head_dim), or (B, heads, T, head_dim) with
     ``heads_first``; in1: the same fp32 table as :func:`rope_header` takes, (T, head_dim/2, 2) of
-    (cos, sin).  With ``heads_at_launch`` the head count is read from ``sideband_value``.
+    (cos, sin).  With ``heads_at_launch`` the head count is read from ``sideband_value``; with
+    ``positions`` a token's table row is an int32 read from the sideband pointer, one per token
+    of the flattened (B, T) axes, as in :func:`rope_header`.
     head_dim/2 must be a power-of-two number of 16-byte vectors (bf16 / fp16: head_dim = 16, 32,
     64, 128, 256, 512; fp32: 8 ... 256), so that a head never straddles a 64-lane wave.
     """
@@ -192,15 +202,18 @@ def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", b
         raise ValueError("head_dim/2 must be a power-of-two multiple (1..32) of %d elements for %s" % (vec, dtype))
     if heads_at_launch and heads_first:
         raise ValueError("with heads_first the head count is not needed: leave heads_at_launch off")
-    name = "sideaware_rope_half_%s_%s_%s_t%d_h%s_d%d" % (
-        "bwd" if backward else "fwd", dtype, "bhtd" if heads_first else "bthd", T,
+    if positions and heads_first:
+        raise ValueError("positions are per token of a (B, T, heads, head_dim) tensor")
+    name = "sideaware_rope_half_%s_%s_%s_t%s_h%s_d%d" % (
+        "bwd" if backward else "fwd", dtype, "bhtd" if heads_first else "bthd", "pos" if positions else str(T),
         "N" if heads_at_launch else str(n_heads), head_dim)
+    heads_expr = "(size_type)val" if heads_at_launch else "rope_heads"
     if heads_first:
         token = "(int)(row % rope_T)"
-    elif heads_at_launch:
-        token = "(int)((row / (size_type)val) % rope_T)"
+    elif positions:
+        token = "mem[row / %s]" % heads_expr
     else:
-        token = "(int)((row / rope_heads) % rope_T)"
+        token = "(int)((row / %s) %% rope_T)" % heads_expr
     # forward: first half x1*c - x2*s, second half x2*c + x1*s; backward: the signs swap
     keep_sign, send_sign = ("-", "+") if backward else ("+", "-")
     lines = ["#define KERNEL_NAME %s\n" % name,
@@ -256,7 +269,7 @@ def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", b
         "    const bool second = in_head >= rope_half;\n"
         "    const int pair = (second ? in_head - rope_half + rope_vec / 2 : in_head);   // first pair this lane rotates\n"
         "    idx_i0 = vec_idx;\n"
-        "    idx_i1 = (size_type)((token * rope_half + pair) / (rope_vec / 2));       // in units of rope_vec floats\n"
+        "    idx_i1 = (size_type)(((size_type)token * rope_half + pair) / (rope_vec / 2));   // in units of rope_vec floats\n"
         "    idx_i2 = 0;\n"
         "    idx_i3 = 0;\n"
         "    return false;\n"

@@ -61,8 +61,14 @@ def freqs_cis_table(head_dim: int, end: int, theta: float, use_scaled: bool = Fa
 _ROPE_DTYPES = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
 
 
+def _check_positions(positions: torch.Tensor, tokens: int) -> None:
+    assert positions.dtype == torch.int32 and positions.is_cuda and positions.is_contiguous(), \
+        "positions are a contiguous int32 device tensor"
+    assert positions.numel() == tokens, "one position per token of the flattened (B, T) axes"
+
+
 def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q: int, n_kv: int,
-          layout: str, backward: bool) -> torch.Tensor:
+          layout: str, backward: bool, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     assert x.dim() == 4, "activations are (B, T, heads, head_dim)"
     B, T, heads, head_dim = x.shape
     if layout == "qkv":
@@ -72,7 +78,13 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
     dtype = _ROPE_DTYPES.get(x.dtype)
     if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
-    assert freqs.dtype == torch.float32 and freqs.shape == (T, head_dim)
+    if positions is None:
+        assert freqs.dtype == torch.float32 and freqs.shape == (T, head_dim)
+    else:
+        assert layout == "heads", "positions go with separate q / k tensors"
+        assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
+        _check_positions(positions, B * T)
+        T = 0                                   # the sequence length is not part of the compiled text
     if out is None:
         out = x
     else:
@@ -81,11 +93,12 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
             # value heads are skipped by the kernel (neither read nor written): out of place they
             # have to be carried over by a copy first
             torch.ops.sideaware.memcpy(out, x)
-    key = (T, n_q, n_kv, head_dim, dtype, layout, backward)
+    key = (T, n_q, n_kv, head_dim, dtype, layout, backward, positions is not None)
     kid = _kernel_ids.get(key)
     if kid is None:
-        kid = _kernel(key, lambda: headers.rope_header(T, n_q, n_kv, head_dim, dtype, layout, backward))
-    _elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+        kid = _kernel(key, lambda: headers.rope_header(max(T, 1), n_q, n_kv, head_dim, dtype, layout, backward,
+                                                       positions=positions is not None))
+    _elementwise(kid, out, None, None, None, x, freqs, None, None, positions, 0, 0, 0)
     return out
 
 
@@ -99,13 +112,16 @@ def rope_backward_qkv(dout, freqs, n_q: int, n_kv: int, out=None):
     return _rope(dout, freqs, out, n_q, n_kv, "qkv", True)
 
 
-def rope_forward_heads(x, freqs, out=None):
-    """(B, T, heads, head_dim), every head rotated: one call per separate q or k tensor."""
-    return _rope(x, freqs, out, 0, 0, "heads", False)
+def rope_forward_heads(x, freqs, out=None, positions=None):
+    """(B, T, heads, head_dim), every head rotated: one call per separate q or k tensor.
+    ``positions``: an int32 device tensor with one table row number per token of the flattened
+    (B, T) axes, for decoding steps and packed sequences (``freqs`` then has a row for every
+    position that occurs); without it token t of every sequence uses row t."""
+    return _rope(x, freqs, out, 0, 0, "heads", False, positions)
 
 
-def rope_backward_heads(dout, freqs, out=None):
-    return _rope(dout, freqs, out, 0, 0, "heads", True)
+def rope_backward_heads(dout, freqs, out=None, positions=None):
+    return _rope(dout, freqs, out, 0, 0, "heads", True, positions)
 
 
 class _Segment(ctypes.Structure):
@@ -131,10 +147,12 @@ def elementwise_batch(kernel_id: int, segments) -> None:
     wrapper.library().sideaware_elementwise_batch(kernel_id, len(arr), arr, device, stream)
 
 
-def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool):
+def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool, positions: Optional[torch.Tensor] = None):
     first = tensors[0]
     assert first.dim() == 4, "activations are (B, T, heads, head_dim)"
     T, head_dim = first.shape[1], first.shape[3]
+    if positions is not None:
+        return _rope_many_at_positions(tensors, freqs, backward, positions, half=False)
     dtype = _ROPE_DTYPES.get(first.dtype)
     if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
@@ -147,18 +165,40 @@ def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool):
     return tensors
 
 
-def rope_forward_heads_many(tensors, freqs):
+def _rope_many_at_positions(tensors, freqs, backward: bool, positions: torch.Tensor, half: bool):
+    first = tensors[0]
+    B, T, head_dim = first.shape[0], first.shape[1], first.shape[3]
+    dtype = _ROPE_DTYPES.get(first.dtype)
+    if dtype is None:
+        raise TypeError("RoPE storage is float32, bfloat16 or float16")
+    assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
+    _check_positions(positions, B * T)
+    for t in tensors:
+        assert t.dim() == 4 and t.is_contiguous() and t.shape[:2] == first.shape[:2] and t.shape[3] == head_dim \
+            and t.dtype == first.dtype
+    key = ("rope_many_at_positions", head_dim, dtype, backward, half)
+    if half:
+        make = lambda: headers.rope_half_header(1, 0, head_dim, dtype, backward, heads_at_launch=True, positions=True)
+    else:
+        make = lambda: headers.rope_header(1, 0, 0, head_dim, dtype, "heads", backward, heads_at_launch=True, positions=True)
+    kid = _kernel(key, make)
+    elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], positions, t.shape[2]) for t in tensors])
+    return tensors
+
+
+def rope_forward_heads_many(tensors, freqs, positions=None):
     """Rotates several (B, T, heads, head_dim) tensors in place in ONE launch: q and k of a
-    grouped-query model (different head counts, same T, head_dim and dtype) share a grid."""
-    return _rope_heads_many(list(tensors), freqs, False)
+    grouped-query model (different head counts, same T, head_dim and dtype) share a grid.
+    ``positions`` as in :func:`rope_forward_heads`."""
+    return _rope_heads_many(list(tensors), freqs, False, positions)
 
 
-def rope_backward_heads_many(tensors, freqs):
-    return _rope_heads_many(list(tensors), freqs, True)
+def rope_backward_heads_many(tensors, freqs, positions=None):
+    return _rope_heads_many(list(tensors), freqs, True, positions)
 
 
 def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], heads_first: bool,
-               backward: bool) -> torch.Tensor:
+               backward: bool, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     assert x.dim() == 4 and x.is_contiguous(), "activations are contiguous (B, T, heads, head_dim) or (B, heads, T, head_dim)"
     if heads_first:
         _, heads, T, head_dim = x.shape
@@ -167,32 +207,42 @@ def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor]
     dtype = _ROPE_DTYPES.get(x.dtype)
     if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
-    assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    if positions is None:
+        assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
+    else:
+        assert not heads_first, "positions are per token of a (B, T, heads, head_dim) tensor"
+        assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
+        _check_positions(positions, x.shape[0] * T)
+        T = 1                                   # the sequence length is not part of the compiled text
     if out is None:
         out = x
     assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
-    key = ("rope_half", T, heads, head_dim, dtype, heads_first, backward)
-    kid = _kernel(key, lambda: headers.rope_half_header(T, heads, head_dim, dtype, backward, heads_first))
-    _elementwise(kid, out, None, None, None, x, freqs, None, None, None, 0, 0, 0)
+    key = ("rope_half", T, heads, head_dim, dtype, heads_first, backward, positions is not None)
+    kid = _kernel(key, lambda: headers.rope_half_header(T, heads, head_dim, dtype, backward, heads_first,
+                                                        positions=positions is not None))
+    _elementwise(kid, out, None, None, None, x, freqs, None, None, positions, 0, 0, 0)
     return out
 
 
-def rope_half_forward(x, freqs, out=None, heads_first: bool = False):
+def rope_half_forward(x, freqs, out=None, heads_first: bool = False, positions=None):
     """RoPE for the half-split pair layout (element i of a head pairs with element
     i + head_dim/2, the "rotate_half" convention): (B, T, heads, head_dim), or
     (B, heads, T, head_dim) with ``heads_first``.  ``freqs`` is the same (T, head_dim) table the
-    interleaved ops take ([t, 2i] = cos, [t, 2i+1] = sin of pair i).  In place unless ``out`` is given."""
-    return _rope_half(x, freqs, out, heads_first, False)
+    interleaved ops take ([t, 2i] = cos, [t, 2i+1] = sin of pair i).  In place unless ``out`` is given.
+    ``positions`` as in :func:`rope_forward_heads`."""
+    return _rope_half(x, freqs, out, heads_first, False, positions)
 
 
-def rope_half_backward(dout, freqs, out=None, heads_first: bool = False):
-    return _rope_half(dout, freqs, out, heads_first, True)
+def rope_half_backward(dout, freqs, out=None, heads_first: bool = False, positions=None):
+    return _rope_half(dout, freqs, out, heads_first, True, positions)
 
 
-def rope_half_forward_many(tensors, freqs, backward: bool = False):
+def rope_half_forward_many(tensors, freqs, backward: bool = False, positions=None):
     """Half-split RoPE of several (B, T, heads, head_dim) tensors in place in ONE launch (q and k
-    of a grouped-query model)."""
+    of a grouped-query model).  ``positions`` as in :func:`rope_forward_heads`."""
     tensors = list(tensors)
+    if positions is not None:
+        return _rope_many_at_positions(tensors, freqs, backward, positions, half=True)
     first = tensors[0]
     T, head_dim = first.shape[1], first.shape[3]
     dtype = _ROPE_DTYPES.get(first.dtype)

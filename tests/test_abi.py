@@ -395,3 +395,18 @@ def test_half_split_rope_headers_compile_and_refuse_heads_that_would_straddle_a_
     for bad in ((96, "bf16"), (24, "fp32"), (1024, "fp32"), (7, "fp32")):           # 6 lanes, 3 lanes, 128 lanes, odd
         with pytest.raises(ValueError):
             headers.rope_half_header(16, 2, bad[0], bad[1])
+
+
+def test_rope_headers_with_per_token_positions_compile(lib):
+    for header in (headers.rope_header(1, 32, 0, 128, "bf16", "heads", positions=True),
+                   headers.rope_header(1, 0, 0, 64, "fp32", "heads", backward=True, heads_at_launch=True, positions=True),
+                   headers.rope_half_header(1, 8, 128, "bf16", positions=True),
+                   headers.rope_half_header(1, 0, 128, "fp16", heads_at_launch=True, positions=True)):
+        assert b"mem[row" in header
+        for variant in (0, 3, 4):
+            rc, log = compile_ok(lib, header, variant)
+            assert rc == 0, log
+    with pytest.raises(ValueError):
+        headers.rope_header(16, 4, 2, 64, "fp32", "qkv", positions=True)          # packed QKV has no positions form
+    with pytest.raises(ValueError):
+        headers.rope_half_header(16, 4, 64, "bf16", heads_first=True, positions=True)

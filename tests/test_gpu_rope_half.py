@@ -139,3 +139,73 @@ def test_batched_launches_replay_from_a_hip_graph(sa):
         assert np.array_equal(bits(q), want_q) and np.array_equal(bits(k), want_k), trial
         assert np.array_equal(bits(q2), want_q2) and np.array_equal(bits(k2), want_k2), trial
     assert_no_library_error(sa)
+
+
+# --------------------------------------------------------------------------------------- positions
+
+def _rows(table, positions):
+    """The table a flattened (1, B*T, heads, D) run of the oracle needs: row i = the row of token i."""
+    return np.ascontiguousarray(table[positions.reshape(-1)])
+
+
+@pytest.mark.parametrize("B,T,H,D", [(3, 5, 4, 64), (16, 1, 32, 128), (2, 129, 3, 128)])
+def test_rope_at_given_positions_vs_oracle_both_pair_layouts(sa, B, T, H, D):
+    # decoding steps and packed sequences: each token names its own table row
+    from l2_torch_alloc_amd import ops
+    max_pos = 1000
+    table = O.freqs_cis(D, max_pos, 500000.0)
+    freqs = torch.from_numpy(table).cuda()
+    g = torch.Generator().manual_seed(B * 100 + T)
+    pos = torch.randint(0, max_pos, (B, T), generator=g, dtype=torch.int32)
+    x = torch.randn(B, T, H, D, generator=g).to(torch.bfloat16)
+    flat = bits(x).reshape(1, B * T, H, D)
+    rows = _rows(table, pos.numpy())
+    want_pairs = O.rope_forward_heads_bf16(flat, rows).reshape(B, T, H, D)
+    want_half = O.rope_half_forward_heads_bf16(flat, rows).reshape(B, T, H, D)
+    pos_d = pos.cuda()
+    y = ops.rope_forward_heads(x.cuda(), freqs, positions=pos_d)
+    z = ops.rope_half_forward(x.cuda(), freqs, positions=pos_d)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(y), want_pairs)
+    assert np.array_equal(bits(z), want_half)
+    # positions 0..T-1 in every sequence are the plain op
+    plain = torch.arange(T, dtype=torch.int32).repeat(B, 1).cuda()
+    if T <= max_pos:
+        a = ops.rope_forward_heads(x.cuda(), freqs, positions=plain)
+        b = ops.rope_forward_heads(x.cuda(), freqs[:T].contiguous())
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(a), bits(b))
+
+
+def test_q_and_k_at_given_positions_in_one_launch_and_backward(sa):
+    from l2_torch_alloc_amd import ops
+    B, T, D, max_pos = 4, 7, 128, 300
+    table = O.freqs_cis(D, max_pos, 10000.0)
+    freqs = torch.from_numpy(table).cuda()
+    g = torch.Generator().manual_seed(77)
+    pos = torch.randint(0, max_pos, (B, T), generator=g, dtype=torch.int32)
+    rows = _rows(table, pos.numpy())
+    q0 = torch.randn(B, T, 8, D, generator=g)
+    k0 = torch.randn(B, T, 2, D, generator=g)
+    for half in (False, True):
+        q, k = q0.cuda(), k0.cuda()
+        fwd = O.rope_half_forward_heads_f32 if half else O.rope_forward_heads_f32
+        bwd = O.rope_half_backward_heads_f32 if half else O.rope_backward_heads_f32
+        if half:
+            ops.rope_half_forward_many([q, k], freqs, positions=pos.cuda())
+        else:
+            ops.rope_forward_heads_many([q, k], freqs, positions=pos.cuda())
+        torch.cuda.synchronize()
+        assert_no_library_error(sa)
+        want_q = fwd(q0.numpy().reshape(1, B * T, 8, D), rows)
+        want_k = fwd(k0.numpy().reshape(1, B * T, 2, D), rows)
+        assert np.array_equal(bits(q).reshape(want_q.shape), want_q.view(np.uint32))
+        assert np.array_equal(bits(k).reshape(want_k.shape), want_k.view(np.uint32))
+        if half:
+            ops.rope_half_forward_many([q, k], freqs, backward=True, positions=pos.cuda())
+        else:
+            ops.rope_backward_heads_many([q, k], freqs, positions=pos.cuda())
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(q).reshape(want_q.shape), bwd(want_q, rows).view(np.uint32))
+        assert np.array_equal(bits(k).reshape(want_k.shape), bwd(want_k, rows).view(np.uint32))
