@@ -11,6 +11,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <ctime>
+#include <atomic>
 #include <fstream>
 #include <mutex>
 
@@ -117,7 +118,9 @@ bool read_file(const std::string& path, std::vector<char>& out) {
 }
 
 void write_file_atomic(const std::string& path, const std::vector<char>& data) {
-    std::string tmp = path + ".tmp" + std::to_string((long)::getpid());
+    // a name of its own per writer: two threads of one process may compile the same text at once
+    static std::atomic<unsigned long> serial{0};
+    std::string tmp = path + ".tmp" + std::to_string((long)::getpid()) + "_" + std::to_string(serial.fetch_add(1));
     {
         std::ofstream f(tmp, std::ios::binary);
         if (!f) return;
