@@ -256,11 +256,11 @@ def sideaware_elementwise(kernel_id: int,
     # The byte count is taken from out0, as the reference does (test.py:114-116).
     num_bytes = out0.numel() * out0.element_size() if out0 is not None else 0
     assert num_bytes > 0
-    device, stream = _device_and_stream(out0)
+    o0, o1, o2, o3 = _check(out0, "out0"), _check(out1, "out1"), _check(out2, "out2"), _check(out3, "out3")
+    i0, i1, i2, i3 = _check(in0, "in0"), _check(in1, "in1"), _check(in2, "in2"), _check(in3, "in3")
+    device, stream = _device_and_stream(out0)            # after the checks: out0 is on a GPU
     (_lib or library()).sideaware_elementwise(
-        kernel_id, num_bytes,
-        _check(out0, "out0"), _check(out1, "out1"), _check(out2, "out2"), _check(out3, "out3"),
-        _check(in0, "in0"), _check(in1, "in1"), _check(in2, "in2"), _check(in3, "in3"),
+        kernel_id, num_bytes, o0, o1, o2, o3, i0, i1, i2, i3,
         sideband_tensor.data_ptr() if sideband_tensor is not None else 0, sideband_value,
         parallel_chunks, forced_sm_per_side, device, stream)
 
