@@ -717,3 +717,43 @@ def test_input_only_op_with_sideband_result(sa, n_ints):
     assert int(acc[1]) == n_ints // 4
     want = (3 * int(x.sum(dtype=torch.int64))) & 0xffffffff
     assert (int(acc[0]) & 0xffffffff) == want
+
+
+NARROW_HEADER = """
+typedef %(out)s o0;
+typedef %(inp)s i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = (o0)(in0 + (i0)sideband);
+}
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {1,0,0,0};
+"""
+
+
+@pytest.mark.parametrize("inp,out,tin,tout,per_lane", [
+    ("double", "unsigned char", torch.float64, torch.uint8, 2),     # 2 elements per lane: 2-byte stores
+    ("double", "short", torch.float64, torch.int16, 4),             # 4-byte stores
+    ("float", "unsigned char", torch.float32, torch.uint8, 4),      # 4-byte stores
+    ("float", "short", torch.float32, torch.int16, 8),              # 8-byte stores
+    ("short", "double", torch.int16, torch.float64, 64),            # four 16-byte stores per lane
+])
+def test_outputs_narrower_and_wider_than_the_input(sa, inp, out, tin, tout, per_lane):
+    # every store width of the template: 2, 4, 8 and several times 16 bytes per lane, in both
+    # cache classes, with a partial last tile and guard elements behind the output
+    lib = sa.library()
+    stream = torch.cuda.current_stream().cuda_stream
+    kid = sa.sideaware_create_kernel((NARROW_HEADER % {"inp": inp, "out": out}).encode())
+    wide_bytes = max(torch.empty(0, dtype=tin).element_size(), torch.empty(0, dtype=tout).element_size())
+    for n in (16 // wide_bytes * 5, 4096 * 3 + 16 // wide_bytes * 7, (300 << 20) // wide_bytes):
+        x = (torch.arange(n, dtype=torch.int64, device="cuda") % 97).to(tin)
+        y = torch.full((n + 64,), 7, dtype=tout, device="cuda")
+        lib.sideaware_elementwise(kid, n * wide_bytes, y.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, 0, 3, 0, 0, 0, stream)
+        torch.cuda.synchronize()
+        assert_no_library_error(sa)
+        assert torch.equal(y[:n], (x + 3).to(tout)), (inp, out, n)
+        assert bool((y[n:] == 7).all()), (inp, out, n)
+    del per_lane
