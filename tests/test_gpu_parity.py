@@ -757,3 +757,43 @@ def test_outputs_narrower_and_wider_than_the_input(sa, inp, out, tin, tout, per_
         assert torch.equal(y[:n], (x + 3).to(tout)), (inp, out, n)
         assert bool((y[n:] == 7).all()), (inp, out, n)
     del per_lane
+
+
+FOUR_BY_FOUR_HEADER = b"""
+typedef float o0; typedef short o1; typedef double o2; typedef unsigned char o3;
+typedef float i0; typedef int i1; typedef short i2; typedef unsigned char i3;
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = in0 + (float)in1;
+    out1 = (short)(in2 + in3);
+    out2 = (double)in0 * 2.0 + (double)sideband;
+    out3 = (unsigned char)(in3 ^ (unsigned char)(element_idx & 0xff));
+}
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {1,0,1,0};
+"""
+
+
+@pytest.mark.parametrize("n", [4, 1024 * 7 + 12, 5 * (1 << 20)])
+def test_four_inputs_and_four_outputs_of_four_widths(sa, n):
+    # the widest arrays (float in0, double out2 is wider still) set the vector: 16 bytes of the
+    # wider of (i0, o0), so 4 elements per lane; out2 then takes 32 bytes per lane, out3 four
+    kid = sa.sideaware_create_kernel(FOUR_BY_FOUR_HEADER)
+    g = torch.Generator().manual_seed(n)
+    in0 = torch.randint(-1000, 1000, (n,), generator=g).float().cuda()
+    in1 = torch.randint(-1000, 1000, (n,), generator=g, dtype=torch.int32).cuda()
+    in2 = torch.randint(-1000, 1000, (n,), generator=g, dtype=torch.int16).cuda()
+    in3 = torch.randint(0, 200, (n,), generator=g, dtype=torch.uint8).cuda()
+    out0 = torch.zeros(n, dtype=torch.float32, device="cuda")
+    out1 = torch.zeros(n, dtype=torch.int16, device="cuda")
+    out2 = torch.zeros(n, dtype=torch.float64, device="cuda")
+    out3 = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    torch.ops.sideaware.elementwise(kid, out0, out1, out2, out3, in0, in1, in2, in3, None, 5, 0, 0)
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    idx = (torch.arange(n, device="cuda") & 0xff).to(torch.uint8)
+    assert torch.equal(out0, in0 + in1.float())
+    assert torch.equal(out1, in2 + in3.to(torch.int16))
+    assert torch.equal(out2, in0.double() * 2.0 + 5.0)
+    assert torch.equal(out3, in3 ^ idx)
