@@ -24,6 +24,9 @@ CASES = {
     "rope_fp32_qkv_scaled": (1, 8, 2, 2, 64, 10000.0, True, "fp32", "qkv"),
     "rope_fp32_heads_gpt2": (1, 5, 12, 0, 64, 10000.0, False, "fp32", "heads"),
     "rope_bf16_heads_llama3": (1, 7, 8, 0, 128, 500000.0, False, "bf16", "heads"),
+    # the half-split pair layout (element i pairs with element i + HS/2), every head rotated
+    "rope_half_fp32_heads": (2, 5, 3, 0, 32, 10000.0, False, "fp32", "half"),
+    "rope_half_bf16_heads_llama3": (1, 6, 8, 0, 128, 500000.0, False, "bf16", "half"),
 }
 
 
@@ -39,13 +42,16 @@ def make(name):
         if layout == "qkv":
             out["y"] = O.rope_forward_qkv_f32(x, freqs, Nq, Nkv)
             out["dx"] = O.rope_backward_qkv_f32(out["y"], freqs, Nq, Nkv)
+        elif layout == "half":
+            out["y"] = O.rope_half_forward_heads_f32(x, freqs)
+            out["dx"] = O.rope_half_backward_heads_f32(out["y"], freqs)
         else:
             out["y"] = O.rope_forward_heads_f32(x, freqs)
             out["dx"] = O.rope_backward_heads_f32(out["y"], freqs)
     else:
         xb = O.f32_to_bf16(x)
         out["x"] = xb
-        out["y"] = O.rope_forward_heads_bf16(xb, freqs)
+        out["y"] = O.rope_half_forward_heads_bf16(xb, freqs) if layout == "half" else O.rope_forward_heads_bf16(xb, freqs)
     return out
 
 

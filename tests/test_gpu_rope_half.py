@@ -209,3 +209,21 @@ def test_q_and_k_at_given_positions_in_one_launch_and_backward(sa):
         torch.cuda.synchronize()
         assert np.array_equal(bits(q).reshape(want_q.shape), bwd(want_q, rows).view(np.uint32))
         assert np.array_equal(bits(k).reshape(want_k.shape), bwd(want_k, rows).view(np.uint32))
+
+
+def test_committed_golden_vectors(sa):
+    import os
+    from l2_torch_alloc_amd import ops
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    g = np.load(os.path.join(golden, "rope_half_fp32_heads.npz"))
+    freqs = torch.from_numpy(g["freqs"]).cuda()
+    y = ops.rope_half_forward(torch.from_numpy(g["x"]).cuda(), freqs)
+    dx = ops.rope_half_backward(y.clone(), freqs)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), g["y"].view(np.uint32)) and np.array_equal(bits(dx), g["dx"].view(np.uint32))
+    g = np.load(os.path.join(golden, "rope_half_bf16_heads_llama3.npz"))
+    x = torch.from_numpy(g["x"].view(np.int16).copy()).view(torch.bfloat16).cuda()
+    y = ops.rope_half_forward(x, torch.from_numpy(g["freqs"]).cuda())
+    torch.cuda.synchronize()
+    assert_no_library_error(sa)
+    assert np.array_equal(bits(y), g["y"])
