@@ -54,3 +54,28 @@ def test_registry_tuning_and_compiler_under_thread_sanitizer(tmp_path):
     assert proc.returncode == 0, proc.stderr[-4000:]
     out = run(exe)
     assert "bad=0" in out
+
+
+def test_registry_and_compiler_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    # the same driver, host code only, for memory errors instead of races: the registry, the ELF
+    # symbol reader of the run-time compiler, the configuration text, the error slot
+    hipcc = shutil.which("hipcc") or os.path.join(sa_build.rocm_root(), "bin", "hipcc")
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    sa_build.generate_template_literal()
+    exe = str(tmp_path / "registry_asan")
+    lib_dir = os.path.join(sa_build.rocm_root(), "lib")
+    cmd = [hipcc, "--offload-arch=gfx950", "-std=c++17", "-O1", "-g",
+           "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-pthread",
+           os.path.join(NATIVE, "registry_tsan_main.cpp")] + \
+          [os.path.join(CSRC, s) for s in sa_build.SOURCES] + \
+          ["-L" + lib_dir, "-lhiprtc", "-Wl,-rpath," + lib_dir, "-o", exe]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-4000:]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", UBSAN_OPTIONS="print_stacktrace=1",
+               SIDEAWARE_NO_DISK_CACHE="1")
+    run_ = subprocess.run([exe], capture_output=True, text=True, timeout=900, env=env)
+    assert "AddressSanitizer" not in run_.stderr and "runtime error" not in run_.stderr, run_.stderr[-6000:]
+    assert run_.returncode == 0 and "bad=0" in run_.stdout, (run_.returncode, run_.stdout[-2000:], run_.stderr[-4000:])
