@@ -3,8 +3,9 @@
 Two drivers: the allocator's policy code over the fake backing store with six threads allocating,
 freeing, trimming and reading statistics on one pool; and the library's own translation units
 (registry, tuning knobs, configuration setters, error slot, run-time compiler) with six threads
-registering headers, changing knobs and compiling at once through the C ABI.  No GPU is involved:
-neither driver makes a device call that needs one.
+registering headers, changing knobs and compiling at once through the C ABI.  The second driver
+also runs under AddressSanitizer and UBSan.  No GPU is involved: neither driver makes a device
+call that needs one.
 """
 import os
 import shutil
