@@ -80,3 +80,15 @@ def test_registry_and_compiler_under_address_and_undefined_behaviour_sanitizers(
     run_ = subprocess.run([exe], capture_output=True, text=True, timeout=900, env=env)
     assert "AddressSanitizer" not in run_.stderr and "runtime error" not in run_.stderr, run_.stderr[-6000:]
     assert run_.returncode == 0 and "bad=0" in run_.stdout, (run_.returncode, run_.stdout[-2000:], run_.stderr[-4000:])
+
+
+def test_pool_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    # the allocator's policy code with the same six-thread driver, for memory errors
+    exe = str(tmp_path / "pool_asan")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+                    "-pthread", os.path.join(NATIVE, "pool_tsan_main.cpp"), os.path.join(CSRC, "pool.cpp"), "-o", exe],
+                   check=True, capture_output=True, text=True)
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=900,
+                          env=dict(os.environ, UBSAN_OPTIONS="print_stacktrace=1"))
+    assert "AddressSanitizer" not in proc.stderr and "runtime error" not in proc.stderr, proc.stderr[-6000:]
+    assert proc.returncode == 0 and "bad=0 live=0 backing_used=0" in proc.stdout, (proc.returncode, proc.stdout[-2000:])
