@@ -593,13 +593,14 @@ struct SegmentArgs {
     int tail_block;
     unsigned int first_block;
 };
-struct BatchArgs {
-    SegmentArgs seg[kMaxSegments];
+struct BatchArgs {                        // the batched entry point's arguments, in their order
     unsigned int count;
     unsigned int blocks_end[kMaxSegments];
     unsigned int reserved;
+    SegmentArgs seg[kMaxSegments];
 };
-static_assert(sizeof(SegmentArgs) == 128 && sizeof(BatchArgs) == 128 * kMaxSegments + 8 + 4 * kMaxSegments,
+static_assert(sizeof(SegmentArgs) == 128 && sizeof(BatchArgs) == 128 * kMaxSegments + 8 + 4 * kMaxSegments &&
+              offsetof(BatchArgs, seg) == 40 && kMaxSegments == 8,
               "the device side declares the same layout");
 
 // The instantiation a launch over these arrays needs.  Index width: 32-bit below 2 GiB, 64-bit from
@@ -775,29 +776,30 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
                                         slots_wanted_for(ctx, k, entry->default_groups, parallel_groups, forced_per_side, t));
 
     // The kernel's arguments, laid out as the device code declares them (natural alignment, in
-    // order) and handed to the runtime as one block.
-    struct Args32 { int nv; void* p[9]; int val; int ft, b0, uc, run; unsigned int r; int tail; };
-    struct Args64 { long long nv; void* p[9]; int val; long long ft, b0, uc, run; unsigned int r; int tail; };
-    static_assert(offsetof(Args32, tail) == 104 && offsetof(Args64, tail) == 124, "kernel argument layout");
+    // order: the plan's scalars, the workgroup count, then i0, o0 and the other pointers) and
+    // handed to the runtime as one block.
+    struct Args32 { int nv, ft, b0, uc, run; unsigned int r; int tail; int val; unsigned int blocks; void* p[9]; };
+    struct Args64 { long long nv, ft, b0, uc, run; unsigned int r; int tail; int val; unsigned int blocks; void* p[9]; };
+    static_assert(offsetof(Args32, p) == 40 && sizeof(Args32) == 112 && offsetof(Args64, p) == 56 && sizeof(Args64) == 128,
+                  "kernel argument layout");
     union { Args32 a32; Args64 a64; } args;
     size_t args_bytes;
-    void* const ptrs[9] = {out0, out1, out2, out3, (void*)in0, (void*)in1, (void*)in2, (void*)in3, sideband_memory};
+    void* const ptrs[9] = {(void*)in0, out0, out1, out2, out3, (void*)in1, (void*)in2, (void*)in3, sideband_memory};
     if (wide) {
         Args64& a = args.a64;
         a.nv = num_vectors;
-        std::memcpy(a.p, ptrs, sizeof ptrs);
-        a.val = sideband_value;
         a.ft = plan.full_tiles; a.b0 = plan.b0; a.uc = plan.u_count; a.run = plan.run;
-        a.r = plan.r; a.tail = plan.tail_block;
-        args_bytes = offsetof(Args64, tail) + sizeof(int);
+        a.r = plan.r; a.tail = plan.tail_block; a.val = sideband_value; a.blocks = plan.grid;
+        std::memcpy(a.p, ptrs, sizeof ptrs);
+        args_bytes = sizeof(Args64);
     } else {
         Args32& a = args.a32;
         a.nv = (int)num_vectors;
-        std::memcpy(a.p, ptrs, sizeof ptrs);
-        a.val = sideband_value;
         a.ft = (int)plan.full_tiles; a.b0 = (int)plan.b0; a.uc = (int)plan.u_count; a.run = (int)plan.run;
-        a.r = plan.r; a.tail = plan.tail_block;
-        args_bytes = offsetof(Args32, tail) + sizeof(int);
+        a.r = plan.r; a.tail = plan.tail_block; a.val = sideband_value; a.blocks = plan.grid;
+        std::memset((char*)&a + 36, 0, 4);                       // the padding in front of the pointers
+        std::memcpy(a.p, ptrs, sizeof ptrs);
+        args_bytes = sizeof(Args32);
     }
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &args_bytes, HIP_LAUNCH_PARAM_END};
 
@@ -883,10 +885,11 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
             set_error("elementwise_batch: %llu workgroups do not fit one grid", blocks);
             return;
         }
-        void* args[1] = {&batch};
+        size_t batch_bytes = sizeof batch;
+        void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &batch, HIP_LAUNCH_PARAM_BUFFER_SIZE, &batch_bytes, HIP_LAUNCH_PARAM_END};
         ScopedDevice guard(ctx->device);
         hipError_t err = hipModuleLaunchKernel(k->fn_batch, (unsigned)blocks, 1, 1, (unsigned)k->wg_threads, 1, 1, 0,
-                                               (hipStream_t)stream, args, nullptr);
+                                               (hipStream_t)stream, nullptr, extra);
         if (err != hipSuccess) {
             set_error("elementwise_batch: launch of kernel %d failed: %s", kernel_id, hipGetErrorString(err));
             (void)hipGetLastError();

@@ -39,7 +39,7 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
                 return c > next ? next : c;
             };
             const long long lo = cut(s), n = cut(s + 1) - lo;
-            sa_segment_args& a = batch.seg[s];
+            sa_segment_args& a = batch.segments.seg[s];
             a.output0 = o0 ? o0 + lo : nullptr; a.output1 = o1 ? o1 + lo : nullptr;
             a.output2 = o2 ? o2 + lo : nullptr; a.output3 = o3 ? o3 + lo : nullptr;
             a.input0 = i0 ? i0 + lo : nullptr; a.input1 = i1 ? i1 + lo : nullptr;
@@ -61,7 +61,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             for (unsigned t = 0; t < SA_WG_THREADS; t++) {
                 blockIdx = {b, 0, 0};
                 threadIdx = {t, 0, 0};
-                SA_CONCAT(KERNEL_NAME, _batch)(batch);
+                const unsigned* e = batch.blocks_end;
+                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments);
             }
         }
         return;
@@ -75,9 +76,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
         for (unsigned t = 0; t < SA_WG_THREADS; t++) {
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
-            KERNEL_NAME(nv, o0, o1, o2, o3, i0, i1, i2, i3, mem, val,
-                                  (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
-                                  p.r, p.tail_block);
+            KERNEL_NAME(nv, (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
+                        p.r, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem);
         }
     }
 }
