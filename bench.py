@@ -312,7 +312,7 @@ def bench_rope_bf16(steps, warmup, main_figure_only=False, prewarm=0):
         lib.sideaware_elementwise_batch(kid_half, 2, batches[counter[0] % sets], 0, stream)
         counter[0] += 1
 
-    sec_half = time_region(step_half, steps, warmup + sets)
+    sec_half = time_region(step_half, steps, warmup + sets + prewarm)     # the cold-cache part before it let the clocks drop
     del scrub, qk, batches
 
     # for scale: the same step in eager PyTorch (complex multiply in fp32, back to bf16), out of place
