@@ -36,8 +36,8 @@ from bench_util import GiB, HBM_PEAK_GBPS, MiB, _abi, gbps, log, time_each, time
 # the runtime's own 256 MiB buffer copy in the same run (FETCH_SIZE reads 131083.5 KiB for
 # 262144 KiB fetched, so x1.99983; WRITE_SIZE reads 262144.0, so x1.0).
 TRAFFIC_PROFILE = "profiles/sideaware_copy_256MiB_and_rope_bf16_llama3_hbm_traffic.txt"
-COPY_256MIB_TRAFFIC_BYTES = int((131084.0 * 1.99983 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
-ROPE_STEP_TRAFFIC_BYTES = int((165785.0 * 1.99983 + 327680.0) * 1024)         # 675.0 MB, 1.0028 x algorithmic (q and k in one launch)
+COPY_256MIB_TRAFFIC_BYTES = int((131082.5 * 1.99983 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
+ROPE_STEP_TRAFFIC_BYTES = int((165782.5 * 1.99983 + 327680.0) * 1024)         # 675.0 MB, 1.0028 x algorithmic (q and k in one launch)
 
 
 # ------------------------------------------------------------------------------------- workloads
