@@ -750,12 +750,17 @@ def test_outputs_narrower_and_wider_than_the_input(sa, inp, out, tin, tout, per_
     wide_bytes = max(torch.empty(0, dtype=tin).element_size(), torch.empty(0, dtype=tout).element_size())
     for n in (16 // wide_bytes * 5, 4096 * 3 + 16 // wide_bytes * 7, (300 << 20) // wide_bytes):
         x = (torch.arange(n, dtype=torch.int64, device="cuda") % 97).to(tin)
-        y = torch.full((n + 64,), 7, dtype=tout, device="cuda")
-        lib.sideaware_elementwise(kid, n * wide_bytes, y.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, 0, 3, 0, 0, 0, stream)
-        torch.cuda.synchronize()
-        assert_no_library_error(sa)
-        assert torch.equal(y[:n], (x + 3).to(tout)), (inp, out, n)
-        assert bool((y[n:] == 7).all()), (inp, out, n)
+        # the output on a 64-byte boundary (write-through stores) and 16 bytes past one (the
+        # instantiation with the compiler's stores)
+        for shift in (0, 16 // torch.empty(0, dtype=tout).element_size()):
+            y = torch.full((n + 64 + shift,), 7, dtype=tout, device="cuda")
+            out_view = y[shift:]
+            lib.sideaware_elementwise(kid, n * wide_bytes, out_view.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, 0, 3, 0, 0, 0,
+                                      stream)
+            torch.cuda.synchronize()
+            assert_no_library_error(sa)
+            assert torch.equal(out_view[:n], (x + 3).to(tout)), (inp, out, n, shift)
+            assert bool((out_view[n:] == 7).all()) and bool((y[:shift] == 7).all()), (inp, out, n, shift)
     del per_lane
 
 
