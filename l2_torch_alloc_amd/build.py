@@ -14,8 +14,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "sideaware.so")
 
-SOURCES = ["sideaware.hip", "pool.cpp", "hip_backing.cpp", "rtc.cpp"]
-DEPENDS = SOURCES + ["pool.h", "hip_backing.h", "rtc.h", "elementwise_kernel.hip.inc",
+SOURCES = ["sideaware.hip", "side_map.hip", "pool.cpp", "hip_backing.cpp", "rtc.cpp"]
+DEPENDS = SOURCES + ["pool.h", "hip_backing.h", "rtc.h", "side_map.h", "launch_plan.h", "elementwise_kernel.hip.inc",
                      os.path.join("..", "..", "include", "sideaware.h")]
 
 

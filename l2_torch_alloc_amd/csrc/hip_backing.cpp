@@ -45,12 +45,17 @@ void* HipBacking::acquire(size_t bytes) {
         }
         aligned = (void*)(((uintptr_t)raw + kRegionAlign - 1) / kRegionAlign * kRegionAlign);
     }
-    std::lock_guard<std::mutex> lk(mu_);
-    raw_of_[aligned] = raw;
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        raw_of_[aligned] = raw;
+    }
+    // which half of the device holds which granule of the new arena (a few timed loads)
+    sides_.add_arena(aligned, bytes);
     return aligned;
 }
 
 void HipBacking::release(void* ptr, size_t) {
+    sides_.remove_arena(ptr);
     void* raw = ptr;
     {
         std::lock_guard<std::mutex> lk(mu_);
@@ -64,6 +69,16 @@ void HipBacking::release(void* ptr, size_t) {
     if (hipFree(raw) != hipSuccess) {
         std::fprintf(stderr, "sideaware: hipFree(%p) failed: %s\n", raw, hipGetErrorString(hipGetLastError()));
     }
+}
+
+// Where in the free run [lo, hi) a block of `bytes` should start so that its granules alternate
+// between the device's halves the same way every other block's do; 0 when nothing is known about
+// the arena the run lies in.
+uintptr_t HipBacking::place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) {
+    uintptr_t base = 0;
+    unsigned int flip = 0;
+    if (!sides_.arena_of((const void*)lo, &base, &flip)) return 0;
+    return canonical_start(sides_.hash(), flip, base, lo, hi, bytes);
 }
 
 void HipBacking::sync_device() {

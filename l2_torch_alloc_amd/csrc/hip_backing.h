@@ -5,20 +5,26 @@
 #include <unordered_map>
 
 #include "pool.h"
+#include "side_map.h"
 
 namespace sideaware {
 
 class HipBacking final : public Backing {
 public:
-    explicit HipBacking(int device) : device_(device) {}
+    explicit HipBacking(int device) : device_(device), sides_(device) {}
     void* acquire(size_t bytes) override;
     void release(void* ptr, size_t bytes) override;
     void sync_device() override;
     void order_after(void* producer, void* consumer) override;
     int free_foreign(void* ptr, void* stream) override;
+    uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) override;
+
+    // What was measured about the arenas handed to the pool (side_map.h).
+    SideRegistry& sides() { return sides_; }
 
 private:
     int device_;
+    SideRegistry sides_;
     std::mutex mu_;
     // aligned pointer handed to the pool -> pointer hipMalloc returned (they differ only when
     // the runtime did not return a 2 MiB-aligned address by itself)

@@ -111,21 +111,46 @@ void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
     ix.by_size.emplace(e.bytes, addr);
 }
 
-// Takes `bytes` from the front of the best-fitting free extent; the remainder stays free.
-bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken) {
+// Takes `bytes` from the best-fitting free extent; what is left of it stays free.  Normally the
+// block is the extent's front.  With `canonical` the backing store is asked where in the extent the
+// block should start so that the device's memory halves alternate through it like through every
+// other block placed this way (Backing::place_canonical); the first few extents in best-fit order
+// are tried, and when none can hold such a block (or the backing store knows no rule) the front of
+// the best fit is taken after all.
+bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken, bool canonical) {
     ExtentIndex& ix = free_[kind];
     auto sit = ix.by_size.lower_bound({bytes, 0});
     if (sit == ix.by_size.end()) return false;
-    *addr = sit->second;
-    auto ait = ix.by_addr.find(*addr);
+    uintptr_t start = sit->second;
+    if (canonical) {
+        int tries = 0;
+        for (auto cand = sit; cand != ix.by_size.end() && tries < kCanonicalTries; ++cand, ++tries) {
+            const uintptr_t at = backing_->place_canonical(cand->second, cand->second + cand->first, bytes);
+            if (at == 0) continue;
+            assert(at >= cand->second && at + bytes <= cand->second + cand->first && at % kRegionAlign == 0);
+            sit = cand;
+            start = at;
+            st_.canonical_placements++;
+            break;
+        }
+    }
+    const uintptr_t ext_addr = sit->second;
+    auto ait = ix.by_addr.find(ext_addr);
     *taken = ait->second;
+    *addr = start;
     ix.by_size.erase(sit);
     ix.by_addr.erase(ait);
-    if (taken->bytes > bytes) {
+    if (start > ext_addr) {
+        Extent front = *taken;
+        front.bytes = start - ext_addr;
+        ix.by_addr[ext_addr] = front;
+        ix.by_size.emplace(front.bytes, ext_addr);
+    }
+    if (ext_addr + taken->bytes > start + bytes) {
         Extent rest = *taken;
-        rest.bytes = taken->bytes - bytes;
-        ix.by_addr[*addr + bytes] = rest;
-        ix.by_size.emplace(rest.bytes, *addr + bytes);
+        rest.bytes = ext_addr + taken->bytes - (start + bytes);
+        ix.by_addr[start + bytes] = rest;
+        ix.by_size.emplace(rest.bytes, start + bytes);
     }
     (kind == kSlabArenas ? st_.bytes_free_slab_arena : st_.bytes_free_arena) -= bytes;
     return true;
@@ -137,7 +162,7 @@ bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* t
 void* Pool::carve_locked(size_t rounded, void* stream) {
     uintptr_t addr;
     Extent e;
-    if (!extent_take_locked(kLargeArenas, rounded, &addr, &e)) return nullptr;
+    if (!extent_take_locked(kLargeArenas, rounded, &addr, &e, rounded >= kCanonicalMinBytes)) return nullptr;
     if (e.freed_on.overflow) {
         backing_->sync_device();
         st_.device_syncs++;
@@ -163,9 +188,18 @@ void* Pool::carve_locked(size_t rounded, void* stream) {
 // give the configured size any more.
 bool Pool::new_arena_locked(int kind, size_t min_bytes) {
     size_t configured = kind == kSlabArenas ? std::min(arena_bytes_, kMaxSlabArenaBytes) : arena_bytes_;
-    size_t want = std::max(configured, min_bytes);
+    // a region that gets an arena of its own still needs room to start on the right page parity
+    size_t padded = min_bytes;
+    if (kind == kLargeArenas && arena_bytes_ != 0 && min_bytes >= kCanonicalMinBytes && min_bytes + kCanonicalSlack > configured) {
+        padded = min_bytes + kCanonicalSlack;
+    }
+    size_t want = std::max(configured, padded);
     void* p = backing_acquire_locked(want);
-    if (!p && want > min_bytes) {
+    if (!p && want > padded) {
+        want = padded;
+        p = backing_acquire_locked(want);
+    }
+    if (!p && padded > min_bytes) {
         want = min_bytes;
         p = backing_acquire_locked(want);
     }
@@ -338,9 +372,9 @@ void* Pool::slab_memory_locked(size_t bytes, Arena** arena) {
     }
     uintptr_t addr;
     Extent e;
-    if (!extent_take_locked(kSlabArenas, bytes, &addr, &e)) {
+    if (!extent_take_locked(kSlabArenas, bytes, &addr, &e, false)) {
         if (!new_arena_locked(kSlabArenas, bytes)) return nullptr;
-        if (!extent_take_locked(kSlabArenas, bytes, &addr, &e)) return nullptr;
+        if (!extent_take_locked(kSlabArenas, bytes, &addr, &e, false)) return nullptr;
     }
     *arena = e.arena;
     return (void*)addr;

@@ -49,6 +49,13 @@ constexpr size_t kSmallGranule = 512;            // alignment and minimum size o
 constexpr size_t kMaxSlabBytes = 64ull << 20;
 constexpr size_t kDefaultArenaBytes = 4ull << 30;
 constexpr size_t kMaxSlabArenaBytes = 1ull << 30;
+// Large regions from this size on are placed where the backing store says the device's memory
+// halves alternate through them in the common pattern (Backing::place_canonical): the arrays an
+// elementwise kernel reads and writes then have the same half at the same offset.  Smaller ones
+// are not worth the 2 MiB hole such a placement can leave in front of them.
+constexpr size_t kCanonicalMinBytes = 32ull << 20;
+constexpr size_t kCanonicalSlack = 2 * kRegionAlign;
+constexpr int kCanonicalTries = 8;
 
 // Where the bytes come from.  The HIP implementation lives in hip_backing.cpp.
 class Backing {
@@ -66,6 +73,11 @@ public:
     virtual void order_after(void* producer, void* consumer) = 0;
     // A pointer the pool never handed out: forward to the runtime's own free.
     virtual int free_foreign(void* ptr, void* stream) = 0;
+    // Where inside the free run [lo, hi) of an arena a block of `bytes` should start so that the
+    // device's memory halves ("sides") alternate through it as they do through every other block
+    // placed this way: a multiple of kRegionAlign in [lo, hi - bytes], or 0 for "anywhere" (no
+    // rule known, or the run cannot hold such a block).
+    virtual uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) { (void)lo; (void)hi; (void)bytes; return 0; }
 };
 
 struct PoolStats {
@@ -93,6 +105,7 @@ struct PoolStats {
     uint64_t bytes_free_slab_arena = 0;  // free extents inside the slabs' arenas
     uint64_t cache_folds = 0;       // times the reuse cache was folded back to serve a request without the driver
     uint64_t refused_frees = 0;     // frees of addresses inside the pool that are not live blocks (double frees, interior pointers)
+    uint64_t canonical_placements = 0;   // large regions placed by the backing store's side rule
 };
 constexpr int kPoolStatsFields = sizeof(PoolStats) / sizeof(uint64_t);
 
@@ -197,7 +210,7 @@ private:
     void* allocate_small_locked(size_t bytes, void* stream);
     void* carve_locked(size_t rounded, void* stream);
     void extent_insert_locked(int kind, uintptr_t addr, Extent e);
-    bool extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken);
+    bool extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken, bool canonical);
     bool new_arena_locked(int kind, size_t min_bytes);
     void flush_cache_locked();
     size_t release_free_arenas_locked(int kind, size_t down_to, bool device_idle = false);

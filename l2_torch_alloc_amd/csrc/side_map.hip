@@ -1,0 +1,351 @@
+#include "side_map.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+
+namespace sideaware {
+
+// ---------------------------------------------------------------------------------------------
+// Measurement
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+constexpr int kProbeLoads = 4;              // timed loads per sample; the first also pays for the address translation
+constexpr size_t kScrubBytes = 128ull << 20;   // read after the first pass: four times the XCDs' L2s together
+constexpr int kProbeGroups = 8;             // one workgroup per XCD, whatever the dealing offset
+
+// Lane 0 of each workgroup times single loads, one at a time, inside the granule at base +
+// offsets[i]: every XCD and every repeat has a 128-byte line of its own (line 8 * repeat + XCD of the
+// granule's 64), so no load is answered by a line another one brought in, and the XCDs walk the
+// samples in different rotations, so they do not queue up behind each other at one memory channel.
+// The fastest repeat after the first (which also pays for the address translation) is kept.
+// lat is [16][n], indexed by the XCD the workgroup found itself on.
+__global__ __launch_bounds__(64) void sa_side_probe(const char* base, const uint64_t* offsets, int n, unsigned int* lat) {
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    xcc &= 0xfu;
+    if (threadIdx.x != 0) return;
+    int acc = 0;
+    const int start = (int)(((unsigned long long)(xcc & 7u) * (unsigned)n) / 8u);
+    for (int step = 0; step < n; step++) {
+        const int i = (start + step) % n;
+        unsigned int best = ~0u;
+        for (int k = 0; k < kProbeLoads; k++) {
+            const int* ptr = (const int*)(base + offsets[i] + (size_t)(k * 8 + (int)(xcc & 7u)) * 128);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            unsigned long long t0 = __builtin_amdgcn_s_memtime();
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t0) :: "memory");
+            int v;
+            asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(ptr) : "memory");
+            unsigned long long t1 = __builtin_amdgcn_s_memtime();
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t1) :: "memory");
+            acc ^= v;
+            const unsigned int d = (unsigned int)(t1 - t0);
+            if (k > 0 && d < best) best = d;
+        }
+        lat[(size_t)xcc * n + i] = best;
+    }
+    if (acc == 0x12345678) lat[0] = (unsigned int)acc;      // keeps the loads alive
+}
+
+// Reads `vectors` 16-byte vectors once: pushes whatever the XCDs' L2s held out of them.
+typedef int sa_probe_v4i __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void sa_side_scrub(const sa_probe_v4i* p, size_t vectors, unsigned int* sink) {
+    sa_probe_v4i acc = {0, 0, 0, 0};
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < vectors; i += (size_t)gridDim.x * 256) acc ^= p[i];
+    if ((acc.x ^ acc.y) == 0x5a5a5a5a && (acc.z ^ acc.w) == 0x5a5a5a5a && acc.x == acc.z) sink[0] = 1;
+}
+
+struct DeviceGuard {
+    int prev = -1;
+    bool switched = false;
+    explicit DeviceGuard(int want) {
+        if (hipGetDevice(&prev) == hipSuccess && prev != want) switched = hipSetDevice(want) == hipSuccess;
+    }
+    ~DeviceGuard() { if (switched) (void)hipSetDevice(prev); }
+};
+
+// A thread that is capturing a stream in the global mode may not launch on another stream: the
+// probe switches the thread to the relaxed mode for its own launches.
+struct RelaxedCapture {
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    bool exchanged = false;
+    RelaxedCapture() { exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess; if (!exchanged) (void)hipGetLastError(); }
+    ~RelaxedCapture() { if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode); }
+};
+
+bool side_debug() {
+    static const bool on = [] { const char* v = std::getenv("SIDEAWARE_SIDE_DEBUG"); return v && v[0] == '1'; }();
+    return on;
+}
+
+bool side_probing_enabled() {
+    const char* v = std::getenv("SIDEAWARE_SIDE_PROBE");
+    return !(v && v[0] == '0');
+}
+
+}  // namespace
+
+SideRegistry::~SideRegistry() {
+    // device buffers, the stream and the pinned slots live until the process ends: launches that
+    // report into the slots may still be queued
+}
+
+// Times loads at base + offsets[i] from every XCD and says, for each i, which half of the XCDs is
+// nearer: 0 (XCDs 0 .. n/2-1), 1, or -1 when the two halves do not differ clearly.
+bool SideRegistry::measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides) {
+    const int n = (int)offsets.size();
+    sides->assign(n, -1);
+    if (n == 0 || n > kMaxProbe || bytes < kScrubBytes) return false;
+    DeviceGuard dev(device_);
+    RelaxedCapture relaxed;
+    if (!probe_stream_) {
+        hipStream_t s = nullptr;
+        if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) { (void)hipGetLastError(); return false; }
+        probe_stream_ = s;
+        if (hipMalloc((void**)&probe_offsets_, kMaxProbe * sizeof(uint64_t)) != hipSuccess ||
+            hipMalloc((void**)&probe_lat_, (16 * kMaxProbe + 16) * sizeof(unsigned int)) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+    }
+    if (!probe_offsets_ || !probe_lat_) return false;
+    hipStream_t st = (hipStream_t)probe_stream_;
+    std::vector<unsigned int> lat(16 * (size_t)n);
+    bool ok = hipMemcpyAsync(probe_offsets_, offsets.data(), n * sizeof(uint64_t), hipMemcpyHostToDevice, st) == hipSuccess;
+    // Two passes with a sweep through the start of the region after each: the first pass brings the
+    // sampled lines into the memory-side cache (so the second times the fabric, not DRAM), the
+    // sweep pushes them out of the XCDs' own L2s again (which keep clean lines across kernels and
+    // would answer the second pass themselves).
+    for (int pass = 0; pass < 2 && ok; pass++) {
+        ok = hipMemsetAsync(probe_lat_, 0, 16 * (size_t)n * sizeof(unsigned int), st) == hipSuccess;
+        if (!ok) break;
+        hipLaunchKernelGGL(sa_side_probe, dim3(kProbeGroups), dim3(64), 0, st, base, probe_offsets_, n, probe_lat_);
+        if (pass == 0) {
+            hipLaunchKernelGGL(sa_side_scrub, dim3(2048), dim3(256), 0, st, (const sa_probe_v4i*)base, kScrubBytes / 16,
+                               probe_lat_ + 16 * (size_t)kMaxProbe);
+        }
+        ok = hipGetLastError() == hipSuccess;
+    }
+    ok = ok && hipMemcpyAsync(lat.data(), probe_lat_, lat.size() * sizeof(unsigned int), hipMemcpyDeviceToHost, st) == hipSuccess;
+    ok = ok && hipStreamSynchronize(st) == hipSuccess;
+    if (!ok) { (void)hipGetLastError(); return false; }
+    for (int i = 0; i < n; i++) {
+        // per half of the device, the middle of its XCDs' times (one XCD delayed by something else
+        // then changes nothing)
+        unsigned int v[2][kProbeGroups / 2];
+        int cnt[2] = {0, 0};
+        for (int x = 0; x < kProbeGroups; x++) {
+            const unsigned int t = lat[(size_t)x * n + i];
+            if (t == 0 || t == ~0u) continue;
+            const int h = x / (kProbeGroups / 2);
+            v[h][cnt[h]++] = t;
+        }
+        if (cnt[0] < 3 || cnt[1] < 3) continue;
+        double mid[2];
+        for (int h = 0; h < 2; h++) {
+            std::sort(v[h], v[h] + cnt[h]);
+            mid[h] = cnt[h] == 4 ? 0.5 * (v[h][1] + v[h][2]) : v[h][1];
+        }
+        const double a = mid[0], b = mid[1];
+        const double lo = a < b ? a : b, hi = a < b ? b : a;
+        if (side_debug() && hi - lo < 0.2 * lo) {
+            std::fprintf(stderr, "sideaware: probe %3d at +0x%llx:", i, (unsigned long long)offsets[i]);
+            for (int x = 0; x < kProbeGroups; x++) std::fprintf(stderr, " %u", lat[(size_t)x * n + i]);
+            std::fprintf(stderr, "\n");
+        }
+        if (hi - lo < 0.2 * lo) continue;                 // near ~450 cycles, far ~680: anything closer is noise
+        (*sides)[i] = a < b ? 0 : 1;
+    }
+    return true;
+}
+
+// Which address bits decide the side?  For every candidate bit, a few granules and their partners
+// with that bit flipped: a bit is in the hash when every pair lands on different sides, out of it
+// when none does, and the whole discovery fails on anything in between.
+void SideRegistry::discover_locked() {
+    if (discovered_) return;
+    discovered_ = true;
+    hash_ = SideHash();
+    if (!side_probing_enabled()) return;
+    DeviceGuard dev(device_);
+    int xcds = 0;
+    if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device_) != hipSuccess || xcds != kProbeGroups) {
+        (void)hipGetLastError();
+        if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: %d XCDs, need %d\n", xcds, kProbeGroups);
+        return;
+    }
+    constexpr size_t kBytes = 1ull << 30;
+    constexpr int kLowBit = 12, kHighBit = 29, kPairsPerBit = 8, kPairsNeeded = 5;
+    size_t free_bytes = 0, total = 0;
+    if (hipMemGetInfo(&free_bytes, &total) != hipSuccess || free_bytes < 2 * kBytes) { (void)hipGetLastError(); return; }
+    char* scratch = nullptr;
+    if (hipMalloc((void**)&scratch, kBytes) != hipSuccess) { (void)hipGetLastError(); return; }
+    std::vector<uint64_t> offsets;
+    uint64_t lcg = 0x9e3779b97f4a7c15ull;
+    for (int b = kLowBit; b <= kHighBit; b++) {
+        for (int j = 0; j < kPairsPerBit; j++) {
+            lcg = lcg * 6364136223846793005ull + 1442695040888963407ull;
+            uint64_t x = (lcg >> 20) % kBytes;
+            x &= ~((1ull << kLowBit) - 1) & ~(1ull << b);
+            offsets.push_back(x);
+            offsets.push_back(x | (1ull << b));
+        }
+    }
+    std::vector<int> sides;
+    const bool measured = measure_locked(scratch, kBytes, offsets, &sides);
+    (void)hipFree(scratch);
+    if (!measured) {
+        if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: the probe could not run\n");
+        return;
+    }
+    uint64_t mask = 0;
+    size_t at = 0;
+    for (int b = kLowBit; b <= kHighBit; b++) {
+        int flips = 0, same = 0;
+        for (int j = 0; j < kPairsPerBit; j++, at += 2) {
+            if (sides[at] < 0 || sides[at + 1] < 0) continue;
+            (sides[at] != sides[at + 1] ? flips : same)++;
+        }
+        if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: bit %d: %d pairs flip, %d do not\n", b, flips, same);
+        if (flips >= kPairsNeeded && same == 0) mask |= 1ull << b;
+        else if (!(same >= kPairsNeeded && flips == 0)) return;              // not a parity of address bits
+    }
+    // the kernels assume granules of exactly 8 KiB
+    if (!((mask >> kSideGranuleLog2) & 1) || (mask & ((1ull << kSideGranuleLog2) - 1))) return;
+    hash_.known = true;
+    hash_.address_mask = mask;
+}
+
+void SideRegistry::add_arena(void* base, size_t bytes) {
+    std::lock_guard<std::mutex> g(mu_);
+    discover_locked();
+    ArenaSide a;
+    a.base = (uintptr_t)base;
+    a.bytes = bytes;
+    if (hash_.known && bytes >= (1u << kSidePairLog2) && a.base % (1u << kSidePairLog2) == 0) {
+        // The arena's constant: a vote over granules spread across it.  One sample that
+        // contradicts the others means the arena is not laid out as the hash says.
+        constexpr int kSamples = 48;
+        std::vector<uint64_t> offsets;
+        uint64_t lcg = 0x2545f4914f6cdd1dull ^ (uint64_t)a.base;
+        const uint64_t granules = bytes >> kSideGranuleLog2;
+        for (int i = 0; i < kSamples; i++) {
+            lcg = lcg * 6364136223846793005ull + 1442695040888963407ull;
+            uint64_t gi = i < 8 ? (uint64_t)i * 37 % granules : (lcg >> 17) % granules;
+            if (gi + 1 >= granules && granules > 1) gi = granules - 2;        // the repeats stay inside the arena
+            offsets.push_back(gi << kSideGranuleLog2);
+        }
+        std::vector<int> sides;
+        if (measure_locked((const char*)base, bytes, offsets, &sides)) {
+            int votes[2] = {0, 0};
+            for (int i = 0; i < kSamples; i++) {
+                if (sides[i] < 0) continue;
+                votes[(unsigned)sides[i] ^ side_parity(offsets[i] & hash_.address_mask)]++;
+            }
+            const int valid = votes[0] + votes[1];
+            if (side_debug()) std::fprintf(stderr, "sideaware: arena %p (%zu MiB): votes %d / %d\n", base, bytes >> 20, votes[0], votes[1]);
+            if (valid >= kSamples * 3 / 4 && (votes[0] == 0 || votes[1] == 0)) {
+                a.known = true;
+                a.flip = votes[1] ? 1u : 0u;
+            }
+        }
+    }
+    arenas_.push_back(a);
+}
+
+void SideRegistry::remove_arena(void* base) {
+    std::lock_guard<std::mutex> g(mu_);
+    for (size_t i = 0; i < arenas_.size(); i++) {
+        if (arenas_[i].base == (uintptr_t)base) {
+            arenas_[i] = arenas_.back();
+            arenas_.pop_back();
+            return;
+        }
+    }
+}
+
+SideHash SideRegistry::hash() {
+    std::lock_guard<std::mutex> g(mu_);
+    return hash_;
+}
+
+int SideRegistry::arenas_known() {
+    std::lock_guard<std::mutex> g(mu_);
+    int n = 0;
+    for (const ArenaSide& a : arenas_) n += a.known ? 1 : 0;
+    return n;
+}
+
+bool SideRegistry::lookup(const void* addr, size_t bytes, SideMap* out) {
+    const uintptr_t p = (uintptr_t)addr;
+    std::lock_guard<std::mutex> g(mu_);
+    if (!hash_.known) return false;
+    for (const ArenaSide& a : arenas_) {
+        if (p >= a.base && p - a.base < a.bytes) {
+            if (!a.known || bytes > a.bytes - (p - a.base)) return false;
+            out->origin_address = a.base;
+            out->pair_mask = hash_.pair_mask();
+            out->flip = a.flip;
+            return true;
+        }
+    }
+    return false;
+}
+
+bool SideRegistry::arena_of(const void* addr, uintptr_t* base, unsigned int* flip) {
+    const uintptr_t p = (uintptr_t)addr;
+    std::lock_guard<std::mutex> g(mu_);
+    if (!hash_.known) return false;
+    for (const ArenaSide& a : arenas_) {
+        if (p >= a.base && p - a.base < a.bytes) {
+            if (!a.known) return false;
+            *base = a.base;
+            *flip = a.flip;
+            return true;
+        }
+    }
+    return false;
+}
+
+int SideRegistry::side_of(const void* addr) {
+    uintptr_t base = 0;
+    unsigned int flip = 0;
+    if (!arena_of(addr, &base, &flip)) return -1;
+    const SideHash h = hash();
+    return (int)(side_parity(((uintptr_t)addr - base) & h.address_mask) ^ flip);
+}
+
+unsigned int* SideRegistry::feedback_slot(void* stream, unsigned int* dealing) {
+    std::lock_guard<std::mutex> g(mu_);
+    *dealing = 0;
+    if (!feedback_) {
+        DeviceGuard dev(device_);
+        void* p = nullptr;
+        if (hipHostMalloc(&p, kFeedbackSlots * 64, hipHostMallocMapped) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        std::fill_n((unsigned int*)p, kFeedbackSlots * 16, 0u);
+        feedback_ = (volatile unsigned int*)p;
+    }
+    int slot;
+    auto it = slot_of_stream_.find(stream);
+    if (it != slot_of_stream_.end()) {
+        slot = it->second;
+    } else {
+        // more streams than slots: the late ones share the last slot (and each other's reports)
+        slot = (int)slot_of_stream_.size() < kFeedbackSlots ? (int)slot_of_stream_.size() : kFeedbackSlots - 1;
+        slot_of_stream_.emplace(stream, slot);
+    }
+    volatile unsigned int* word = feedback_ + (size_t)slot * 16;
+    const unsigned int v = *word;
+    if (v & 0x80000000u) *dealing = v & 0xfu;
+    return (unsigned int*)word;
+}
+
+}  // namespace sideaware

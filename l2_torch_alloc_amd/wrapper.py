@@ -70,6 +70,10 @@ _SIGNATURES = {
     "sideaware_arena_bytes": (None, [_sz]),
     "sideaware_num_xcds": (_ci, []),
     "sideaware_xcd_dealing_verified": (_ci, []),
+    "sideaware_side_address_mask": (ctypes.c_ulonglong, []),
+    "sideaware_side_of": (_ci, [_vp]),
+    "sideaware_stream_dealing": (_ci, [_vp]),
+    "sideaware_launch_counts": (None, [ctypes.POINTER(ctypes.c_ulonglong), ctypes.POINTER(ctypes.c_ulonglong)]),
     "sideaware_last_error": (ctypes.c_char_p, []),
     "sideaware_clear_error": (None, []),
     "sideaware_compile_check": (_ci, [ctypes.c_char_p, _ci, ctypes.c_char_p, _sz]),
@@ -89,7 +93,7 @@ POOL_STAT_FIELDS = (
     "backing_releases", "stream_syncs", "device_syncs", "trims", "ladder_retries", "failures",
     "foreign_frees", "bytes_live", "bytes_cached_large", "bytes_cached_small", "bytes_reserved",
     "peak_reserved", "large_carves", "arenas_acquired", "bytes_free_arena", "bytes_free_slab_arena",
-    "cache_folds", "refused_frees",
+    "cache_folds", "refused_frees", "canonical_placements",
 )
 
 

@@ -19,6 +19,23 @@
 
 static unsigned g_stripe_log2 = 14, g_slot_run = 1, g_segments = 1;
 
+// The plan for one array: the striped one, or, in an instantiation built with SA_SIDED, the sided
+// one with an origin, arena constant and dealing offset derived from the case (any values must
+// give a map that visits every tile once).
+static sideaware::LaunchPlan make_plan(unsigned long long base, long long nv, unsigned grid) {
+    if (sa_sided) {
+        sideaware::SideMap side;
+        side.origin_address = ((base * 2654435761ull) >> 7) & ~0x3fffull;
+        side.pair_mask = SA_SIDE_PAIR_MASK;
+        side.flip = (unsigned)(nv & 1);
+        side.dealing = (unsigned)((grid + nv + g_stripe_log2) % SA_NUM_XCD);
+        return sideaware::plan_launch_sided(base, nv, sideaware_kernel_meta[0], SA_NUM_XCD, g_stripe_log2 % 9,
+                                            g_slot_run, grid / SA_NUM_XCD, side);
+    }
+    return sideaware::plan_launch(base, nv, sideaware_kernel_meta[0], SA_NUM_XCD,
+                                  1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
+}
+
 // `grid` is the caller's wish, as the launcher's parallel_groups would be: a persistent grid of
 // that many workgroups (rounded to whole XCDs), or 0 for one workgroup per tile.  The plan is made
 // by the same function the launcher uses.
@@ -47,10 +64,9 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             a.mem = mem; a.val = val; a.num_vectors = n;
             const unsigned long long seg_base = sideaware_kernel_meta[2] ? (unsigned long long)a.output0
                                                                           : (unsigned long long)a.input0;
-            sideaware::LaunchPlan p = sideaware::plan_launch(seg_base, n, sideaware_kernel_meta[0], SA_NUM_XCD,
-                                                             1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
+            sideaware::LaunchPlan p = make_plan(seg_base, n, grid);
             a.full_tiles = p.full_tiles; a.b0 = p.b0; a.u_count = p.u_count; a.run = p.run;
-            a.r = p.r; a.tail_block = p.tail_block; a.first_block = blocks;
+            a.r = p.r_word; a.tail_block = p.tail_block; a.first_block = blocks;
             blocks += p.grid;
             batch.blocks_end[s] = blocks;
         }
@@ -62,14 +78,13 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
                 blockIdx = {b, 0, 0};
                 threadIdx = {t, 0, 0};
                 const unsigned* e = batch.blocks_end;
-                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments);
+                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments, nullptr);
             }
         }
         return;
     }
     const unsigned long long base = sideaware_kernel_meta[2] ? (unsigned long long)o0 : (unsigned long long)i0;
-    sideaware::LaunchPlan p = sideaware::plan_launch(base, (long long)nv, sideaware_kernel_meta[0], SA_NUM_XCD,
-                                                     1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
+    sideaware::LaunchPlan p = make_plan(base, (long long)nv, grid);
     gridDim = {p.grid, 1, 1};
     blockDim = {SA_WG_THREADS, 1, 1};
     for (unsigned b = 0; b < p.grid; b++) {
@@ -77,7 +92,7 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
             KERNEL_NAME(nv, (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
-                        p.r, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem);
+                        p.r_word, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem, nullptr);
         }
     }
 }

@@ -121,6 +121,13 @@ CONFIGS = [
     ("INCREMENT", 0, 2, False),      # the built-in copy's setting
     ("MIXED", 0, None, False),
     ("MIXED", 1, 2, True),
+    # variant bit 5: the sided ownership map (tiles of 4 KiB and of 8 KiB, both index widths, both orders)
+    ("INCREMENT", 32, 1, False),
+    ("INCREMENT", 33, 2, True),
+    ("INCREMENT", 32, 2, False),
+    ("INCREMENT", 33, 1, True),
+    ("MIXED", 32, 1, False),         # o0 is wider than i0: the map follows o0
+    ("INCREMENT", 32, 4, False),     # tiles of 16 KiB cannot be sided: the instantiation falls back to stripes
 ]
 
 
