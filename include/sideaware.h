@@ -180,8 +180,10 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * (1: stores are written through the XCD's private L2; 0: the compiler's write-back stores)
  * (compiled in: after a change every op is compiled afresh on its next launch); "sided" (1: launches
  * whose output lies in an arena of known sides use the sided map, 0: never), "sided_min_bytes" (arrays
- * shorter than this never do) and "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
- * -1: by array size).
+ * shorter than this never do), "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
+ * -1: by array size) and "sided_wrong" (1: sided launches give every XCD the granules of the other half
+ * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,
+ * every access crossing between the dies).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -94,21 +94,23 @@ struct Tuning {
     long long sided = 1;             // 1: launches whose output lies in an arena of known sides use the sided map; 0: never
     long long sided_min_bytes = 8ll << 20;   // ... when the array is at least this long
     long long sided_stripe = -1;     // log2(pairs per stripe of an XCD) of the sided map; -1: by array size
+    long long sided_wrong = 0;       // 1: sided launches give every XCD the granules of the *other* half (an A/B switch)
 };
 
 // The knobs themselves: written by sideaware_tune (and once from the environment), read by every
 // launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
 // a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
-constexpr int kTuneKnobs = 12;
+constexpr int kTuneKnobs = 13;
 static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
                                                    "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd",
-                                                   "write_through", "sided", "sided_min_bytes", "sided_stripe"};
+                                                   "write_through", "sided", "sided_min_bytes", "sided_stripe",
+                                                   "sided_wrong"};
 static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
                                                  "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
                                                  "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD",
                                                  "SIDEAWARE_WRITE_THROUGH", "SIDEAWARE_SIDED", "SIDEAWARE_SIDED_MIN_BYTES",
-                                                 "SIDEAWARE_SIDED_STRIPE"};
-static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}};
+                                                 "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -138,6 +140,7 @@ static Tuning tuning_snapshot() {
     t.sided = g_tune[9].load(std::memory_order_relaxed);
     t.sided_min_bytes = g_tune[10].load(std::memory_order_relaxed);
     t.sided_stripe = g_tune[11].load(std::memory_order_relaxed);
+    t.sided_wrong = g_tune[12].load(std::memory_order_relaxed);
     return t;
 }
 
@@ -170,11 +173,16 @@ static unsigned long long stripe_for(unsigned long long num_bytes, int num_xcds,
 }
 
 // The stripe of the sided map, as log2(pairs of granules an XCD takes in a row).  Measured on MI355X
-// with nothing cache-resident (256 MiB copy: 32 pairs 6.85 TB/s, 4 pairs 6.74, 128 pairs 6.77; 1 GiB:
-// 128 pairs 6.95, 32 pairs 6.90, single pairs 6.86).
-static unsigned int sided_stripe_for(unsigned long long num_bytes, const Tuning& t) {
+// with nothing cache-resident, every setting timed in turn several times over (fractions of 8 TB/s):
+//   copy 64 MiB    16 pairs 0.815, 32 pairs 0.810, 8 pairs 0.812, 128 pairs 0.795
+//   copy 256 MiB   32 pairs 0.865, single pairs 0.860, 64 pairs 0.859, 16 pairs 0.858, 8 pairs 0.837
+//   copy 1 GiB     64 pairs 0.873, 128 pairs 0.870, 32 pairs 0.869, 16 pairs 0.855
+//   bf16 RoPE in place, q (256 MiB) and k (64 MiB) in one launch:
+//                  8 pairs 0.882, 4 pairs 0.881, 16 pairs 0.878, 32 pairs 0.864, 128 pairs 0.842
+static unsigned int sided_stripe_for(unsigned long long num_bytes, bool in_place, const Tuning& t) {
     if (t.sided_stripe >= 0) return (unsigned int)(t.sided_stripe > 12 ? 12 : t.sided_stripe);
-    return num_bytes >= kBigArrayBytes ? 7u : 5u;
+    if (in_place) return 3u;
+    return num_bytes >= kBigArrayBytes ? 6u : num_bytes >= (128ull << 20) ? 5u : 4u;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -696,7 +704,11 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
     if (((uintptr_t)out0 & ((1u << kSideGranuleLog2) - 1)) != 0) return false;
     if (entry->sided_possible.load(std::memory_order_relaxed) == 0) return false;
     if (ctx->num_xcds < 2 || (ctx->num_xcds & (ctx->num_xcds - 1))) return false;
-    return ctx->backing->sides().lookup(out0, num_bytes, map);
+    if (!ctx->backing->sides().lookup(out0, num_bytes, map)) return false;
+    // The counterpart of the reference's FORCE_WRONG_SIDE (sideaware.cu:70-75, 297-298): the same
+    // map with the arena's constant inverted, so that every access crosses to the other half.
+    if (t.sided_wrong) map->flip ^= 1u;
+    return true;
 }
 
 // A sided launch follows its output.  An input that is as wide as the output and read at the
@@ -872,7 +884,7 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     if (k->sided) {
         feedback = ctx->backing->sides().feedback_slot(stream, &side.dealing);
         plan = plan_launch_sided((uint64_t)(uintptr_t)out0, num_vectors, k->tile_vectors, ctx->num_xcds,
-                                 sided_stripe_for(num_bytes, t), t.slot_run, slots_wanted, side);
+                                 sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side);
     } else {
         const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0);
         plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,
@@ -990,7 +1002,7 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
             if (k->sided) {
                 sides[i].dealing = dealing;
                 plan = plan_launch_sided((uint64_t)(uintptr_t)g.out[0], num_vectors, k->tile_vectors, ctx->num_xcds,
-                                         sided_stripe_for(g.num_bytes, t), t.slot_run, slots_wanted, sides[i]);
+                                         sided_stripe_for(g.num_bytes, g.out[0] == g.in[0], t), t.slot_run, slots_wanted, sides[i]);
             } else {
                 const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]);
                 plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,

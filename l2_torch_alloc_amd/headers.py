@@ -45,7 +45,7 @@ _ROPE_TYPES = {
 
 
 def rope_header(T: int, n_q: int, n_kv: int, head_dim: int, dtype: str = "fp32",
-                layout: str = "qkv", backward: bool = False, unrolled: int | None = 2,
+                layout: str = "qkv", backward: bool = False, unrolled: int | None = 1,
                 reverse_order: bool = False, evict_input: bool = True,
                 stream_input: bool | None = None, stream_output: bool | None = None,
                 heads_at_launch: bool = False, positions: bool = False) -> bytes:
@@ -170,7 +170,7 @@ _ROPE_HALF_TYPES = {
 
 
 def rope_half_header(T: int, n_heads: int, head_dim: int, dtype: str = "bf16", backward: bool = False,
-                     heads_first: bool = False, heads_at_launch: bool = False, unrolled: int | None = 2,
+                     heads_first: bool = False, heads_at_launch: bool = False, unrolled: int | None = 1,
                      evict_input: bool = True, positions: bool = False) -> bytes:
     """RoPE for the half-split pair layout ("rotate_half": element i of a head is paired with
     element i + head_dim/2, as Hugging Face / GPT-NeoX style models store q and k), forward or
