@@ -36,8 +36,8 @@ from bench_util import GiB, HBM_PEAK_GBPS, MiB, _abi, gbps, log, time_each, time
 # the runtime's own 256 MiB buffer copy in the same run (FETCH_SIZE reads 131083.5 KiB for
 # 262144 KiB fetched, so x1.99983; WRITE_SIZE reads 262144.0, so x1.0).
 TRAFFIC_PROFILE = "profiles/sideaware_copy_256MiB_and_rope_bf16_llama3_hbm_traffic.txt"
-COPY_256MIB_TRAFFIC_BYTES = int((131082.5 * 1.99983 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
-ROPE_STEP_TRAFFIC_BYTES = int((165782.5 * 1.99983 + 327680.0) * 1024)         # 675.0 MB, 1.0028 x algorithmic (q and k in one launch)
+COPY_256MIB_TRAFFIC_BYTES = int((131084.1 * 1.99983 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
+ROPE_STEP_TRAFFIC_BYTES = int((165813.5 * 1.99983 + 327680.0) * 1024)         # 675.1 MB, 1.0028 x algorithmic (q and k in one launch)
 
 
 # ------------------------------------------------------------------------------------- workloads
@@ -125,7 +125,10 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
     others the same kind of values made on the device; every destination is compared with its
     source afterwards."""
     import torch
-    first = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=torch.Generator().manual_seed(seed)).cuda()
+    if nbytes <= GiB:
+        first = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=torch.Generator().manual_seed(seed)).cuda()
+    else:                                        # too long to make on the host in reasonable time
+        first = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
     srcs = [first] + [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs - 1)]
     dsts = [torch.zeros_like(t) for t in srcs]
     lib, stream = _abi()
@@ -143,6 +146,56 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
     ok = all(bool(torch.equal(d, t)) for d, t in zip(dsts, srcs))
     return {"bytes": nbytes, "pairs": pairs, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec),
             "frac_of_peak": gbps(2 * nbytes, sec) / HBM_PEAK_GBPS, "bit_exact": ok}
+
+
+def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4):
+    """The 256 MiB cycling copy under the three ownership maps, timed in turn `rounds` times over
+    (medians): sided (every XCD moves the granules of its own half of the device), XCD-striped
+    (the map that needs no knowledge of the halves), and sided the wrong way round (every access
+    crosses between the two I/O dies: the reference's FORCE_WRONG_SIDE experiment,
+    sideaware.cu:70-75)."""
+    import ctypes
+    import torch
+    srcs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+    dsts = [torch.zeros_like(t) for t in srcs]
+    lib, stream = _abi()
+    ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
+    counter = [0]
+
+    def launch():
+        d_ptr, s_ptr = ptrs[counter[0] % pairs]
+        counter[0] += 1
+        lib.sideaware_memcpy(d_ptr, s_ptr, nbytes, 0, stream)
+
+    def launches():
+        a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        lib.sideaware_launch_counts(ctypes.byref(a), ctypes.byref(b))
+        return a.value, b.value
+
+    settings = (("sided", 1, 0), ("xcd_striped", 0, 0), ("sided_wrong_way_round", 1, 1))
+    times = {name: [] for name, _, _ in settings}
+    used = {}
+    try:
+        for _ in range(rounds):
+            for name, sided, wrong in settings:
+                lib.sideaware_tune(b"sided", sided)
+                lib.sideaware_tune(b"sided_wrong", wrong)
+                before = launches()
+                times[name].append(time_region(launch, steps, pairs))
+                after = launches()
+                used[name] = "sided map" if after[0] > before[0] else "striped map"
+    finally:
+        lib.sideaware_tune(b"sided", 1)
+        lib.sideaware_tune(b"sided_wrong", 0)
+    ok = all(bool(torch.equal(d, t)) for d, t in zip(dsts, srcs))
+    out = {"bytes": nbytes, "pairs": pairs, "bit_exact": ok,
+           "side_address_mask": hex(lib.sideaware_side_address_mask()),
+           "stream_dealing_offset": lib.sideaware_stream_dealing(stream)}
+    for name, _, _ in settings:
+        sec = statistics.median(times[name])
+        out[name] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes, sec), "frac_of_peak": gbps(2 * nbytes, sec) / HBM_PEAK_GBPS,
+                     "launches_used": used[name]}
+    return out
 
 
 def bench_vendor_copies(nbytes, pairs, steps):
@@ -374,7 +427,7 @@ def bench_other_ops(steps):
     scales = torch.empty(n // 32, dtype=torch.uint8, device="cuda")
     kid = wrapper.sideaware_create_kernel(headers.mxfp8_quantize_header())
     sec = time_region(lambda: lib.sideaware_elementwise(kid, 2 * n, q.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
-                                                        scales.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
+                                                        scales.data_ptr(), n // 8, 0, 0, 0, stream), steps, 3)
     nbytes = 2 * n + n + n // 32
     out["mxfp8_quantize_256MiB_in"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
     kid = wrapper.sideaware_create_kernel(headers.mxfp8_dequantize_header())
@@ -382,6 +435,7 @@ def bench_other_ops(steps):
                                                         scales.data_ptr(), 0, 0, 0, 0, stream), steps, 3)
     out["mxfp8_dequantize_256MiB_out"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
     del x, y, q, scales
+    out["cycling_over_4_buffer_sets"] = bench_other_ops_cycling(steps)
     B, T, NH, HS = 8, 1024, 32, 128
     qkv = torch.randn(B, T, 3 * NH, HS, generator=torch.Generator().manual_seed(7)).cuda()
     freqs = ops.freqs_cis_table(HS, T, 10000.0, True).cuda()
@@ -393,6 +447,47 @@ def bench_other_ops(steps):
                                                             qkv.data_ptr(), freqs.data_ptr(), 0, 0, 0, 0, 0, 0, 0,
                                                             stream), steps, 3)
         out[name] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec)}
+    return out
+
+
+def bench_other_ops_cycling(steps, sets=4):
+    """scale+bias, MXFP8 quantise and dequantise over `sets` distinct groups of buffers in turn
+    (each group 0.4-0.5 GB), so that no launch finds an operand in a cache: the same protocol as
+    the headline copy."""
+    import torch
+    from l2_torch_alloc_amd import headers, wrapper
+    lib, stream = _abi()
+    n = 256 * MiB // 2                                                     # bf16 elements
+    xs = [torch.randn(n, device="cuda").to(torch.bfloat16) for _ in range(sets)]
+    ys = [torch.empty_like(x) for x in xs]
+    qs = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    ss = [torch.empty(n // 32, dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    sb = torch.tensor([1.25, -0.5], dtype=torch.float32, device="cuda")
+    counter = [0]
+
+    def cycle(fn):
+        def step():
+            fn(counter[0] % sets)
+            counter[0] += 1
+        return step
+
+    out = {}
+    kid_sb = wrapper.sideaware_create_kernel(headers.scale_bias_bf16_header())
+    sec = time_region(cycle(lambda i: lib.sideaware_elementwise(kid_sb, 2 * n, ys[i].data_ptr(), 0, 0, 0, xs[i].data_ptr(),
+                                                                0, 0, 0, sb.data_ptr(), 0, 0, 0, 0, stream)), steps, 2 * sets)
+    out["scale_bias_bf16_256MiB"] = {"bytes": 4 * n, "us": sec * 1e6, "GBps": gbps(4 * n, sec),
+                                     "frac_of_peak": gbps(4 * n, sec) / HBM_PEAK_GBPS}
+    nbytes = 2 * n + n + n // 32
+    kid_q = wrapper.sideaware_create_kernel(headers.mxfp8_quantize_header())
+    sec = time_region(cycle(lambda i: lib.sideaware_elementwise(kid_q, 2 * n, qs[i].data_ptr(), 0, 0, 0, xs[i].data_ptr(),
+                                                                0, 0, 0, ss[i].data_ptr(), n // 8, 0, 0, 0, stream)), steps, 2 * sets)
+    out["mxfp8_quantize_256MiB_in"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec),
+                                       "frac_of_peak": gbps(nbytes, sec) / HBM_PEAK_GBPS}
+    kid_d = wrapper.sideaware_create_kernel(headers.mxfp8_dequantize_header())
+    sec = time_region(cycle(lambda i: lib.sideaware_elementwise(kid_d, 2 * n, ys[i].data_ptr(), 0, 0, 0, qs[i].data_ptr(),
+                                                                0, 0, 0, ss[i].data_ptr(), 0, 0, 0, 0, stream)), steps, 2 * sets)
+    out["mxfp8_dequantize_256MiB_out"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": gbps(nbytes, sec),
+                                          "frac_of_peak": gbps(nbytes, sec) / HBM_PEAK_GBPS}
     return out
 
 
@@ -470,11 +565,65 @@ def bench_churn(use_sideaware, n_ops=10000, live_cap=64 * GiB):
             "peak_reserved_bytes": None if use_sideaware else int(torch.cuda.max_memory_reserved())}
 
 
+def bench_churn_raw_calls(n_ops=10000, live_cap=64 * GiB):
+    """The churn's own sequence of allocations and frees (the same seeded sizes, the same two
+    allocations and one free per step, the same dropping of the oldest blocks beyond 64 GiB live)
+    replayed on the C entry points through ctypes, with no tensor, no kernel and no PyTorch in
+    between: what sideaware_malloc_auto / sideaware_free_auto themselves cost when requests miss
+    the exact-size cache and regions are carved."""
+    from l2_torch_alloc_amd import wrapper
+    lib = wrapper.library()
+    sizes = churn_sizes(n_ops)
+    lib.sideaware_oom_raises(0)                  # a null from a ctypes call is checked here, not thrown
+    before = wrapper.sideaware_alloc_stats()
+    live, live_bytes = [], 0
+    t_alloc, t_free = [], []
+    try:
+        for size in sizes:
+            t0 = time.perf_counter_ns()
+            x = lib.sideaware_malloc_auto(size, 0, None)
+            t1 = time.perf_counter_ns()
+            y = lib.sideaware_malloc_auto(size, 0, None)
+            t2 = time.perf_counter_ns()
+            if not x or not y:
+                raise RuntimeError("the pool returned null for %d bytes" % size)
+            t_alloc.append(t1 - t0)
+            t_alloc.append(t2 - t1)
+            t0 = time.perf_counter_ns()
+            lib.sideaware_free_auto(y, size, 0, None)
+            t_free.append(time.perf_counter_ns() - t0)
+            live.append((x, size))
+            live_bytes += size
+            while live_bytes > live_cap:
+                old, old_size = live.pop(0)
+                live_bytes -= old_size
+                t0 = time.perf_counter_ns()
+                lib.sideaware_free_auto(old, old_size, 0, None)
+                t_free.append(time.perf_counter_ns() - t0)
+        for old, old_size in live:
+            lib.sideaware_free_auto(old, old_size, 0, None)
+    finally:
+        lib.sideaware_oom_raises(1)
+    after = wrapper.sideaware_alloc_stats()
+
+    def pct(v, p):
+        v = sorted(v)
+        return v[min(len(v) - 1, int(p * len(v)))] / 1e3
+
+    moved = {k: after[k] - before[k] for k in ("large_hits", "large_carves", "large_misses", "cache_folds", "small_hits",
+                                               "small_carves", "backing_acquires", "canonical_placements")}
+    return {"ops": n_ops, "calls": {"malloc": len(t_alloc), "free": len(t_free)},
+            "alloc_p50_us": pct(t_alloc, 0.50), "alloc_p90_us": pct(t_alloc, 0.90), "alloc_p99_us": pct(t_alloc, 0.99),
+            "free_p50_us": pct(t_free, 0.50), "free_p90_us": pct(t_free, 0.90), "free_p99_us": pct(t_free, 0.99),
+            "pool_events": moved, "peak_reserved_bytes": after["peak_reserved"]}
+
+
 def bench_raw_alloc_calls(n=20000):
     """The C entry points by themselves (ctypes), steady state: alloc+free of one size."""
     from l2_torch_alloc_amd import wrapper
     lib = wrapper.library()
     out = {}
+    lib.sideaware_oom_raises(0)                  # nulls are not expected here, and must not become C++ exceptions
     for label, size in (("small_64KiB", 64 * 1024), ("large_64MiB", 64 * MiB)):
         p = lib.sideaware_malloc_auto(size, 0, None)
         lib.sideaware_free_auto(p, size, 0, None)
@@ -491,6 +640,7 @@ def bench_raw_alloc_calls(n=20000):
         tf.sort()
         out[label] = {"alloc_p50_us": ta[n // 2] / 1e3, "alloc_p99_us": ta[int(n * 0.99)] / 1e3,
                       "free_p50_us": tf[n // 2] / 1e3, "free_p99_us": tf[int(n * 0.99)] / 1e3}
+    lib.sideaware_oom_raises(1)
     return out
 
 
@@ -622,7 +772,9 @@ def main():
     info = wrapper.sideaware_info()
     log("device:", torch.cuda.get_device_name(0), info)
 
-    import bench_experiments as experiments
+    if any((args.stripe_ab, args.inflight_ab, args.cache_probe, args.chain_policy, args.chain_xcd, args.launch_shapes,
+            args.ceiling)):
+        import bench_experiments as experiments      # the sweep modes: not needed by the default run
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": experiments.stripe_ab(args.steps)}))
         return
@@ -669,12 +821,21 @@ def main():
     if not args.quick:
         also["rope_fp32_gpt2"] = bench_rope_fp32_gpt2(200, 10)
         log("rope fp32:", also["rope_fp32_gpt2"])
+        # Every size twice: cycling over enough distinct (src, dst) pairs that the working set is at
+        # least 1 GiB, four times the Infinity Cache (the HBM figure), and one pair in a loop (below
+        # 1 GiB that one is served partly from the Infinity Cache: a cache figure, not an HBM one).
         sweep = {}
-        for label, nbytes, steps in (("4MiB", 4 * MiB, 200), ("64MiB", 64 * MiB, 100), ("256MiB", 256 * MiB, 50),
-                                     ("1GiB", GiB, 20), ("8GiB", 8 * GiB, 5)):
-            sweep[label] = bench_copy(nbytes, steps, 3, "fp32", seed=3)
-            log("sweep", label, sweep[label])
-        also["copy_sweep_fp32_one_pair_in_a_loop"] = sweep
+        for label, nbytes, pairs, steps in (("4MiB", 4 * MiB, 128, 512), ("64MiB", 64 * MiB, 8, 96),
+                                            ("256MiB", 256 * MiB, 8, 48), ("1GiB", GiB, 4, 20), ("8GiB", 8 * GiB, 2, 6)):
+            cycling = bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=3, prewarm=pairs)
+            one_pair = bench_copy(nbytes, steps, 3, "fp32", seed=3)
+            sweep[label] = {"hbm_cycling_pairs": cycling, "one_pair_in_a_loop": one_pair,
+                            "working_set_bytes_cycling": 2 * nbytes * pairs}
+            log("sweep", label, "cycling %.0f GB/s (%.3f)" % (cycling["GBps"], cycling["frac_of_peak"]),
+                "one pair %.0f GB/s" % one_pair["GBps"])
+        also["copy_sweep"] = sweep
+        also["copy_256MiB_ownership_map_ab"] = bench_side_ab()
+        log("ownership map A/B:", also["copy_256MiB_ownership_map_ab"])
         also["copy_4MiB_replayed_from_a_hip_graph"] = bench_small_copy_in_graph()
         log("graph:", also["copy_4MiB_replayed_from_a_hip_graph"])
         also["energy_copy_1GiB"] = bench_energy()
@@ -686,6 +847,9 @@ def main():
         log("vendor copies:", also["vendor_copies_256MiB_rotating_8_pairs"])
         also["alloc_raw_calls"] = bench_raw_alloc_calls()
         log("raw alloc:", also["alloc_raw_calls"])
+        wrapper.library().sideaware_release_unused()
+        also["alloc_churn_raw_entry_points"] = bench_churn_raw_calls()
+        log("churn (raw C entry points, same sequence):", also["alloc_churn_raw_entry_points"])
         wrapper.library().sideaware_release_unused()      # start from an empty pool, like the child process below
         also["alloc_churn_sideaware"] = bench_churn(True)
         also["alloc_churn_sideaware"]["pool"] = wrapper.sideaware_alloc_stats()
@@ -728,7 +892,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": copy["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": copy["GBps"] / HBM_PEAK_GBPS, "traffic": COPY_256MIB_TRAFFIC_BYTES,
                      "traffic_from_profile": TRAFFIC_PROFILE,
-                     "kernel": "sideaware_copy (kernel id 0, 32-bit index, cache-resident class)",
+                     "kernel": "sideaware_copy (kernel id 0, 32-bit index, cache-resident class, sided ownership map)",
                      "algorithmic_bytes_per_launch": 2 * 256 * MiB,
                      "cache_assisted_loop_over_one_pair": None if warm is None else {
                          "achieved": warm["GBps"], "frac": warm["GBps"] / HBM_PEAK_GBPS}},
@@ -736,7 +900,7 @@ def main():
                                "frac": rope["GBps"] / HBM_PEAK_GBPS,
                                "traffic": ROPE_STEP_TRAFFIC_BYTES,
                                "traffic_from_profile": TRAFFIC_PROFILE,
-                               "kernel": "sideaware_rope_fwd_bf16_heads_t4096_hN_0_d128_batch (q and k in one launch)",
+                               "kernel": "sideaware_rope_fwd_bf16_heads_t4096_hN_0_d128_batch (q and k in one launch, sided ownership map)",
                                "algorithmic_bytes_per_launch": rope["bytes"], "ms_per_step": rope["us"] / 1e3},
         "cpu_baseline": cpu,
         "also": also,

@@ -394,7 +394,33 @@ def mxfp8_quantize_header(unrolled: int | None = None) -> bytes:
         "    int shared_exp = (int)((__float_as_uint(amax) >> 23) & 0xff) - 127 - 8;\n"
         "    if (amax == 0.0f || shared_exp < -127) shared_exp = -127;\n"
         "    if (shared_exp > 127) shared_exp = 127;\n"
-        "    if ((vec_idx & 3) == 0) ((unsigned char*)sideband_memory)[vec_idx >> 2] = (unsigned char)(shared_exp + 127);\n"
+        "    // The scale bytes.  A wave's 64 vectors are 16 blocks, 16 consecutive scale bytes: when the\n"
+        "    // whole wave lies inside the array (the launch passes the number of vectors as the sideband\n"
+        "    // value) the bytes of a row of 16 lanes are gathered into one word with row shifts, the four\n"
+        "    // rows' words are read across, and lane 0 writes all 16 bytes with one store, written through\n"
+        "    // the private L2 like the outputs; elsewhere (the last, partial wave; a launch that does not\n"
+        "    // pass the count) every fourth lane stores its own byte.\n"
+        "    const unsigned int sb = (unsigned int)(shared_exp + 127);\n"
+        "    unsigned char *scales = (unsigned char*)sideband_memory;\n"
+        "#if defined(__AMDGCN__)\n"
+        "    if (((vec_idx | 63) < (size_type)sideband_value) && (((size_t)scales & 15) == 0)) {\n"
+        "        unsigned int word = sb;\n"
+        "        word |= (unsigned int)__builtin_amdgcn_update_dpp(0, (int)sb, 0x104, 0xf, 0xf, false) << 8;    // row_shl:4\n"
+        "        word |= (unsigned int)__builtin_amdgcn_update_dpp(0, (int)sb, 0x108, 0xf, 0xf, false) << 16;   // row_shl:8\n"
+        "        word |= (unsigned int)__builtin_amdgcn_update_dpp(0, (int)sb, 0x10C, 0xf, 0xf, false) << 24;   // row_shl:12\n"
+        "        typedef int sa_scale_v4 __attribute__((ext_vector_type(4)));\n"
+        "        sa_scale_v4 all;\n"
+        "        all.x = __builtin_amdgcn_readlane((int)word, 0);\n"
+        "        all.y = __builtin_amdgcn_readlane((int)word, 16);\n"
+        "        all.z = __builtin_amdgcn_readlane((int)word, 32);\n"
+        "        all.w = __builtin_amdgcn_readlane((int)word, 48);\n"
+        "        if ((vec_idx & 63) == 0) {\n"
+        "            sa_scale_v4 *dst = (sa_scale_v4*)(scales + (vec_idx >> 2));\n"
+        "            asm volatile(\"global_store_dwordx4 %0, %1, off sc1\\n\\ts_nop 1\" : : \"v\"(dst), \"v\"(all) : \"memory\");\n"
+        "        }\n"
+        "    } else\n"
+        "#endif\n"
+        "    if ((vec_idx & 3) == 0) scales[vec_idx >> 2] = (unsigned char)sb;\n"
         "    // two conversions fill one 32-bit word with four E4M3 bytes: the second writes the upper half\n"
         "    int words[2] = {0, 0};\n"
         "    #pragma unroll\n"

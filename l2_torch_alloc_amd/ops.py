@@ -281,8 +281,10 @@ def mxfp8_quantize(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Op
     device, stream = wrapper._device_and_stream()
     # num_bytes is the byte length of the wider array, the bf16 input, which the custom-op wrapper
     # cannot know (it sizes the launch from out0, as the reference's does): call the C entry point.
+    # the sideband value is the number of 16-byte vectors: the op gathers a wave's 16 scale bytes
+    # into one store wherever the whole wave lies inside the array
     wrapper.library().sideaware_elementwise(kid, x.numel() * 2, q.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0,
-                                            scales.data_ptr(), 0, 0, 0, device, stream)
+                                            scales.data_ptr(), min(x.numel() // 8, 2 ** 31 - 1), 0, 0, device, stream)
     return q, scales
 
 

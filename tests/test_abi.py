@@ -374,7 +374,9 @@ def test_every_wide_store_is_followed_by_two_wait_states(lib, tmp_path):
     hn = headers.rope_header(4096, 0, 0, 128, "bf16", "heads", heads_at_launch=True)
     fixed = headers.rope_header(4096, 32, 0, 128, "bf16", "heads")
     seen = 0
-    for header, variant in ((None, 0), (None, 2), (None, 3), (None, 12), (hn, 4), (hn, 2), (fixed, 4), (fixed, 10)):
+    quant = headers.mxfp8_quantize_header()          # its op writes a 16-byte store of its own (the scale bytes)
+    for header, variant in ((None, 0), (None, 2), (None, 3), (None, 12), (hn, 4), (hn, 2), (fixed, 4), (fixed, 10),
+                            (None, 32), (hn, 32 + 2), (quant, 0), (quant, 2)):
         lines = [l.strip() for l in _isa_of(lib, tmp_path, header, variant).splitlines()]
         lines = [l.split("//")[0].strip() for l in lines if l and not l.startswith(("//", ";"))]
         for i, l in enumerate(lines):

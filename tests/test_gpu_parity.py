@@ -340,6 +340,33 @@ def test_mxfp8_quantize_vs_oracle(sa):
     want_q, want_s = O.mxfp8_quantize(bits(xh))
     assert np.array_equal(s.cpu().numpy(), want_s)
     assert np.array_equal(q.cpu().numpy(), want_q)
+    # The scale bytes leave through two routes (one 16-byte store per full wave; single bytes in the
+    # last, partial wave, for a scale array off a 16-byte boundary, and for a launch that does not
+    # pass the vector count): lengths around the wave size, a misaligned scale array with guard
+    # bytes, and the raw entry point with sideband value 0.
+    for blocks in (1, 15, 16, 17, 31, 33, 64 + 5, 1024 + 16):
+        m = 32 * blocks
+        x = xh[64:64 + m].clone().cuda()
+        want_q, want_s = O.mxfp8_quantize(bits(xh[64:64 + m].clone()))
+        for shift in (0, 1, 4):
+            pad = torch.full((blocks + 64,), 0xEE, dtype=torch.uint8, device="cuda")
+            scales = pad[16 + shift: 16 + shift + blocks]
+            qq, ss = ops.mxfp8_quantize(x, scales=scales)
+            torch.cuda.synchronize()
+            assert np.array_equal(ss.cpu().numpy(), want_s), (blocks, shift)
+            assert np.array_equal(qq.cpu().numpy(), want_q), (blocks, shift)
+            assert bool((pad[:16 + shift] == 0xEE).all()) and bool((pad[16 + shift + blocks:] == 0xEE).all()), (blocks, shift)
+    lib = sa.library()
+    x = xh[:32 * 200].clone().cuda()
+    want_q, want_s = O.mxfp8_quantize(bits(xh[:32 * 200].clone()))
+    qq = torch.empty(32 * 200, dtype=torch.uint8, device="cuda")
+    ss = torch.empty(200, dtype=torch.uint8, device="cuda")
+    from l2_torch_alloc_amd import headers
+    kid = sa.sideaware_create_kernel(headers.mxfp8_quantize_header())
+    lib.sideaware_elementwise(kid, x.numel() * 2, qq.data_ptr(), 0, 0, 0, x.data_ptr(), 0, 0, 0, ss.data_ptr(), 0, 0, 0, 0,
+                              torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert np.array_equal(ss.cpu().numpy(), want_s) and np.array_equal(qq.cpu().numpy(), want_q)
     # size-independent property at a large size: quantising the dequantised values changes nothing
     big = (torch.randn(64 * MiB // 2, generator=gen) * 3).to(torch.bfloat16).cuda()
     q1, s1 = ops.mxfp8_quantize(big)
