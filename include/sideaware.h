@@ -87,13 +87,18 @@ void sideaware_write_sass(const char* filename);      /* append the gfx950 ISA o
 
 /* ---- queries (sideaware.cu:1492-1522) ---------------------------------------------------- */
 
-/* One byte per CU-sized workgroup slot i of a one-workgroup-per-CU launch:
- * (rank within its XCD << 3) | XCD, the XCD as read from the hardware at start-up. */
+/* The sides are the two halves of an MI355X: each I/O die with its four XCDs and four HBM stacks
+ * (the counterpart of the two L2 sides of the reference's GPUs).  One byte per CU-sized workgroup
+ * slot i of a one-workgroup-per-CU launch, in the reference's layout (sideaware.cu:188, 208-213):
+ * bit 0 is the side of the XCD the slot ran on at start-up, the bits above it the slot's rank among
+ * the slots of that side. */
 void sideaware_fill_side_index(unsigned char* gpu_array);   /* copies num_sms bytes device-to-device */
 const char* sideaware_gpu_side_index(void);                 /* device copy of that table */
 const char* sideaware_cpu_side_index(void);                 /* host copy */
-/* int[5]: { CUs, CUs on XCD 0, CUs on XCD 1, fewest CUs on any XCD, stripe hash | 1<<21 }.
- * The hash has the address bits that choose the owning XCD of a byte in a 2 MiB-aligned region. */
+/* int[5]: { CUs, CUs on side 0, CUs on side 1, the smaller of the two, hash mask }.  The hash mask has
+ * the address bits whose parity, counted from the start of an arena of the pool, says which side
+ * holds a byte (bits 13, 21 and 28 on MI355X: 0x10202000), as measured at start-up; 0 if the device
+ * showed no such structure.  sideaware_side_address_mask() is the same value, 64 bits wide. */
 const int* sideaware_sm_side_summary(void);
 int sideaware_num_sms(void);
 int sideaware_num_sm_side0(void);
@@ -147,6 +152,20 @@ int sideaware_xcd_dealing_verified(void);
  * sideaware_stream_dealing: the XCD that workgroup 0 of the last finished sided launch on `stream`
  * ran on (0 before any): sided launches plan with it.  sideaware_launch_counts: launches so far
  * that used the sided map, and launches that used the XCD-striped one. */
+/* Measures which side `count` sample granules of the device memory [region, region + num_bytes)
+ * lie on, for memory the pool did not hand out (for the pool's own, sideaware_side_of answers
+ * from what was measured when the arena was acquired).  Sample i is the 8 KiB granule number
+ * splitmix64(seed + i) % (num_bytes / 8192), splitmix64(x) being { z = x * 0x9e3779b97f4a7c15 +
+ * 0x9e3779b97f4a7c15; z = (z ^ z >> 30) * 0xbf58476d1ce4e5b9; z = (z ^ z >> 27) * 0x94d049bb133111eb;
+ * z ^ z >> 31 } in 64-bit arithmetic.  One wave on every XCD times single loads inside each sample
+ * granule; `sides[i]` (device memory, `count` ints) receives 0 or 1 for the half of the device whose
+ * XCDs were clearly faster, or -1 where they were not (a few samples in a hundred, at random).
+ * Everything runs on `stream`; the call does not wait.  region must be granule-aligned and num_bytes
+ * at least 128 MiB (that much of the region is read between the probe's two passes, to empty the L2s).
+ * The work space (64 bytes per sample) is allocated and freed in stream order.
+ * Returns 0, or a HIP error code after recording a message for sideaware_last_error. */
+int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
+                          int device, sideaware_stream_t stream);
 unsigned long long sideaware_side_address_mask(void);
 int sideaware_side_of(const void* ptr);
 int sideaware_stream_dealing(sideaware_stream_t stream);

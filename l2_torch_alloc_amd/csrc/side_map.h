@@ -97,6 +97,8 @@ public:
     void add_arena(void* base, size_t bytes);
     void remove_arena(void* base);
 
+    // Measures the hash (once; add_arena does it too if nobody has).
+    void discover();
     SideHash hash();
     // The side map of the arena that holds [addr, addr + bytes), if that arena's constant is known.
     bool lookup(const void* addr, size_t bytes, SideMap* out);
@@ -108,6 +110,11 @@ public:
     // Where workgroup 0 of a sided launch on `stream` reports its XCD (pinned host memory the
     // device can write), and the dealing offset last reported there (0 before the first report).
     unsigned int* feedback_slot(void* stream, unsigned int* dealing);
+
+    // Times loads from every XCD at `count` sample granules of [region, region + bytes) on
+    // `stream` and writes, for each, the side that is clearly nearer (0 or 1), or -1, to the device
+    // array `sides`.  Returns 0, or a negative code for a bad argument (-1) or no memory (-4).
+    int probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream);
 
     // For tests and tools: forget what was measured / pretend.
     void set_hash_for_test(const SideHash& h) { std::lock_guard<std::mutex> g(mu_); hash_ = h; discovered_ = true; }
@@ -121,6 +128,8 @@ private:
         unsigned int flip = 0;
     };
     void discover_locked();
+    int probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream,
+                        unsigned int* work);
     bool measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides);
 
     int device_;

@@ -60,6 +60,80 @@ __global__ __launch_bounds__(256) void sa_side_scrub(const sa_probe_v4i* p, size
     if ((acc.x ^ acc.y) == 0x5a5a5a5a && (acc.z ^ acc.w) == 0x5a5a5a5a && acc.x == acc.z) sink[0] = 1;
 }
 
+// The sample granules of the probe entry points: sample i of a region of `granules` granules is
+// granule splitmix64(seed + i) % granules, so that host and device agree on them without a table.
+__host__ __device__ inline unsigned long long sa_sample_granule(unsigned long long seed, unsigned int i,
+                                                                unsigned long long granules) {
+    unsigned long long z = (seed + (unsigned long long)i) * 0x9e3779b97f4a7c15ull + 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    z ^= z >> 31;
+    return z % granules;
+}
+
+// sa_side_probe with the sample offsets computed on the device (no table to upload).
+__global__ __launch_bounds__(64) void sa_side_probe_seeded(const char* base, unsigned long long granules,
+                                                           unsigned long long seed, int n, unsigned int* lat) {
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    xcc &= 0xfu;
+    if (threadIdx.x != 0) return;
+    int acc = 0;
+    const int start = (int)(((unsigned long long)(xcc & 7u) * (unsigned)n) / 8u);
+    for (int step = 0; step < n; step++) {
+        const int i = (start + step) % n;
+        const unsigned long long offset = sa_sample_granule(seed, (unsigned int)i, granules) << kSideGranuleLog2;
+        unsigned int best = ~0u;
+        for (int k = 0; k < kProbeLoads; k++) {
+            const int* ptr = (const int*)(base + offset + (size_t)(k * 8 + (int)(xcc & 7u)) * 128);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            unsigned long long t0 = __builtin_amdgcn_s_memtime();
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t0) :: "memory");
+            int v;
+            asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(ptr) : "memory");
+            unsigned long long t1 = __builtin_amdgcn_s_memtime();
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t1) :: "memory");
+            acc ^= v;
+            const unsigned int d = (unsigned int)(t1 - t0);
+            if (k > 0 && d < best) best = d;
+        }
+        lat[(size_t)xcc * n + i] = best;
+    }
+    if (acc == 0x12345678) lat[0] = (unsigned int)acc;
+}
+
+// Clears the probe's scratch with a kernel (a memset node recorded into a captured graph is the
+// one thing the graphs of this platform replay wrongly).
+__global__ __launch_bounds__(256) void sa_side_clear(unsigned int* p, int words) {
+    const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (i < words) p[i] = 0;
+}
+
+// One thread per sample: the middle of each half's times, and which half is clearly faster.
+__global__ __launch_bounds__(64) void sa_side_classify(const unsigned int* lat, int n, int* sides) {
+    const int i = (int)(blockIdx.x * 64 + threadIdx.x);
+    if (i >= n) return;
+    float mid[2];
+    bool ok = true;
+    for (int h = 0; h < 2; h++) {
+        unsigned int v[4];
+        int cnt = 0;
+        for (int x = 0; x < 4; x++) {
+            const unsigned int t = lat[(size_t)(h * 4 + x) * n + i];
+            if (t != 0 && t != ~0u) v[cnt++] = t;
+        }
+        if (cnt < 3) { ok = false; break; }
+        for (int a = 1; a < cnt; a++) for (int b = a; b > 0 && v[b] < v[b - 1]; b--) { unsigned int t = v[b]; v[b] = v[b - 1]; v[b - 1] = t; }
+        mid[h] = cnt == 4 ? 0.5f * ((float)v[1] + (float)v[2]) : (float)v[1];
+    }
+    int side = -1;
+    if (ok) {
+        const float lo = mid[0] < mid[1] ? mid[0] : mid[1], hi = mid[0] < mid[1] ? mid[1] : mid[0];
+        if (hi - lo >= 0.2f * lo) side = mid[0] < mid[1] ? 0 : 1;
+    }
+    sides[i] = side;
+}
+
 struct DeviceGuard {
     int prev = -1;
     bool switched = false;
@@ -89,6 +163,54 @@ bool side_probing_enabled() {
 }
 
 }  // namespace
+
+// The probe behind sideaware_probe_sides: everything runs on the
+// caller's stream, the results stay on the device.  `work` holds 16 * count + 16 words.
+int SideRegistry::probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides,
+                                  void* stream, unsigned int* work) {
+    DeviceGuard dev(device_);
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned long long granules = bytes >> kSideGranuleLog2;
+    const int words = 16 * count + 16;
+    for (int pass = 0; pass < 2; pass++) {
+        hipLaunchKernelGGL(sa_side_clear, dim3((words + 255) / 256), dim3(256), 0, st, work, words);
+        hipLaunchKernelGGL(sa_side_probe_seeded, dim3(kProbeGroups), dim3(64), 0, st, (const char*)region, granules, seed,
+                           count, work);
+        if (pass == 0) {
+            hipLaunchKernelGGL(sa_side_scrub, dim3(2048), dim3(256), 0, st, (const sa_probe_v4i*)region, kScrubBytes / 16,
+                               work + 16 * (size_t)count);
+        }
+    }
+    hipLaunchKernelGGL(sa_side_classify, dim3((count + 63) / 64), dim3(64), 0, st, work, count, sides);
+    const hipError_t err = hipGetLastError();
+    return err == hipSuccess ? 0 : (int)err;
+}
+
+int SideRegistry::probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides,
+                              void* stream) {
+    if (!region || !sides || count < 1 || bytes < kScrubBytes || ((uintptr_t)region & ((1u << kSideGranuleLog2) - 1))) return -1;
+    DeviceGuard dev(device_);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned int* work = nullptr;
+    const size_t work_bytes = (16 * (size_t)count + 16) * sizeof(unsigned int);
+    // stream-ordered work space: allocated and given back in the stream's own order, no host wait
+    bool ordered = hipMallocAsync((void**)&work, work_bytes, st) == hipSuccess;
+    if (!ordered) {
+        (void)hipGetLastError();
+        if (hipMalloc((void**)&work, work_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return -4;
+        }
+    }
+    const int rc = probe_on_stream(region, bytes, seed, count, sides, stream, work);
+    if (ordered) {
+        if (hipFreeAsync(work, st) != hipSuccess) (void)hipGetLastError();
+    } else {
+        (void)hipStreamSynchronize(st);
+        (void)hipFree(work);
+    }
+    return rc;
+}
 
 SideRegistry::~SideRegistry() {
     // device buffers, the stream and the pinned slots live until the process ends: launches that
@@ -219,6 +341,11 @@ void SideRegistry::discover_locked() {
     if (!((mask >> kSideGranuleLog2) & 1) || (mask & ((1ull << kSideGranuleLog2) - 1))) return;
     hash_.known = true;
     hash_.address_mask = mask;
+}
+
+void SideRegistry::discover() {
+    std::lock_guard<std::mutex> g(mu_);
+    discover_locked();
 }
 
 void SideRegistry::add_arena(void* base, size_t bytes) {

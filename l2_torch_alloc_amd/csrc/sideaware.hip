@@ -239,14 +239,10 @@ struct DeviceContext {
 static std::once_flag g_devices_once;
 static std::vector<std::unique_ptr<DeviceContext>> g_contexts;
 
-static int stripe_hash_mask(int num_xcds) {
-    // the address bits that select the owning XCD of a byte: log2(num_xcds) bits above the stripe
-    const long long tuned = g_tune[0].load(std::memory_order_relaxed);
-    long long stripe = tuned > 0 ? tuned : kStripeBytes;
-    long long mask = 0;
-    for (long long x = 1; x < num_xcds; x <<= 1) mask |= stripe * x;
-    return (int)(mask & 0x7fffffff);
-}
+// The reference's "hash mask" is the set of address bits whose parity says which L2 side holds a
+// byte (sideaware.cu:1507-1522).  Here: the bits whose parity (counted from the start of an arena)
+// says which half of the device holds it, as the start-up probe found them; 0 when it found none.
+static int side_hash_mask(DeviceContext* ctx);
 
 // Settings may arrive before the first device call: they are kept here, applied to every
 // context that exists, and replayed on contexts created later.
@@ -259,6 +255,11 @@ static size_t g_pending_limit = 0;
 static bool g_have_pending_limit = false;
 static size_t g_pending_arena = 0;
 static bool g_have_pending_arena = false;
+
+static int side_hash_mask(DeviceContext* ctx) {
+    const SideHash h = ctx->backing->sides().hash();
+    return h.known ? (int)(h.address_mask & 0x7fffffff) : 0;
+}
 
 static void apply_config(Pool* pool) {
     std::lock_guard<std::mutex> g(g_config_mu);
@@ -311,13 +312,26 @@ void DeviceContext::initialize() {
 
     int fewest = cus_on_xcd[0];
     for (int x = 1; x < num_xcds; x++) fewest = cus_on_xcd[x] < fewest ? cus_on_xcd[x] : fewest;
+    // The sides are the two halves of the device: XCDs 0 .. n/2-1 and the rest.  The table the
+    // queries hand out has the reference's layout (sideaware.cu:188, 208-213): bit 0 the side of the
+    // slot's XCD, the bits above it the slot's rank among the slots of that side.
+    const int half = num_xcds >= 2 ? num_xcds / 2 : 1;
+    int on_side[2] = {0, 0};
+    for (int i = 0; i < num_cus; i++) {
+        const int x = cpu_side_index[i] & 7;
+        const int side = num_xcds >= 2 ? x / half : 0;
+        cpu_side_index[i] = (unsigned char)(((on_side[side]++ & 0x7f) << 1) | side);
+    }
+    (void)hipMemcpy(gpu_side_index, cpu_side_index, num_cus, hipMemcpyHostToDevice);
+    (void)fewest;
     side_summary[0] = num_cus;
-    side_summary[1] = cus_on_xcd[0];
-    side_summary[2] = num_xcds > 1 ? cus_on_xcd[1] : 0;
-    side_summary[3] = fewest;
-    side_summary[4] = stripe_hash_mask(num_xcds) | (1 << 21);
+    side_summary[1] = on_side[0];
+    side_summary[2] = on_side[1];
+    side_summary[3] = num_xcds >= 2 ? (on_side[0] < on_side[1] ? on_side[0] : on_side[1]) : on_side[0];
 
     backing = std::make_unique<HipBacking>(device);
+    backing->sides().discover();                 // which address bits decide the half of the device (a few ms)
+    side_summary[4] = side_hash_mask(this);
     pool = std::make_unique<Pool>(backing.get());
     // The reference trims its cache from 16 GiB down to 2 GiB on an 80 GB part
     // (sideaware.cu:421-422); keep those proportions of whatever this device holds.
@@ -470,7 +484,7 @@ static std::string config_block(int variant, int num_xcds, int num_cus, const Tu
     s += "#define SA_MAX_SEGMENTS " + std::to_string(kMaxSegments) + "\n";
     // Names the reference injects (sideaware.cu:789-794); kept so headers that mention them compile.
     s += "#define MAX_SM " + std::to_string(num_cus) + "\n";
-    s += "#define HASH " + std::to_string((stripe_hash_mask(num_xcds) | (1 << 21)) / 16) + "\n";
+    s += "#define HASH " + std::to_string(((unsigned long long)side_pair_mask << kSidePairLog2 | (1ull << kSideGranuleLog2)) / 16) + "\n";
     s += "#define SA_BEYOND_CACHE " + std::to_string((variant >> 1) & 1) + "\n";
     s += "#define SA_IN_PLACE " + std::to_string((variant >> 2) & 1) + "\n";
     // the compiler's write-back stores: for outputs off a 64-byte boundary, or when switched to
@@ -1126,7 +1140,6 @@ const int* sideaware_sm_side_summary(void) {
     static int none[5] = {0, 0, 0, 0, 0};
     DeviceContext* ctx = get_context();
     if (!ctx) return none;
-    ctx->side_summary[4] = stripe_hash_mask(ctx->num_xcds) | (1 << 21);
     return ctx->side_summary;
 }
 
@@ -1136,7 +1149,7 @@ int sideaware_num_sm_side1(void) { DeviceContext* c = get_context(); return c ? 
 int sideaware_min_sm_per_side(void) { DeviceContext* c = get_context(); return c ? c->side_summary[3] : 0; }
 int sideaware_hash_mask(void) {
     DeviceContext* c = get_context();
-    return c ? (stripe_hash_mask(c->num_xcds) | (1 << 21)) : 0;
+    return c ? side_hash_mask(c) : 0;
 }
 
 // ---- additions --------------------------------------------------------------------------------
@@ -1161,6 +1174,25 @@ int sideaware_stream_dealing(sideaware_stream_t stream) {
     if (!c) return -1;
     unsigned int dealing = 0;
     return c->backing->sides().feedback_slot(stream, &dealing) ? (int)dealing : -1;
+}
+
+int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
+                          int device, sideaware_stream_t stream) {
+    DeviceContext* c = get_context(device);
+    if (!c) return (int)hipErrorNoDevice;
+    const int rc = c->backing->sides().probe_sides(region, num_bytes, seed, count, sides, stream);
+    if (rc == 0) return 0;
+    if (rc == -1) {
+        set_error("probe_sides: region (%p, granule-aligned), sides (%p), count (%d, at least 1) or num_bytes (%zu, at least "
+                  "128 MiB) is not acceptable", region, (void*)sides, count, num_bytes);
+        return (int)hipErrorInvalidValue;
+    }
+    if (rc == -4) {
+        set_error("probe_sides: no memory for the work space");
+        return (int)hipErrorOutOfMemory;
+    }
+    set_error("probe_sides: launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return rc;
 }
 
 void sideaware_launch_counts(unsigned long long* sided, unsigned long long* striped) {

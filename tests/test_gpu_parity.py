@@ -46,16 +46,21 @@ def test_metadata(sa):
     assert info["num_sms"] == torch.cuda.get_device_properties(0).multi_processor_count
     assert lib.sideaware_num_xcds() >= 1
     assert info["num_sms"] % lib.sideaware_num_xcds() == 0
-    assert info["min"] >= 1 and info["hash"] & (1 << 21)
+    # the sides are the two halves of the device; the hash is what the start-up probe measured
+    assert info["min"] >= 1 and info["hash"] == lib.sideaware_hash_mask() == lib.sideaware_side_address_mask()
+    assert info["hash"] == 0 or info["hash"] & (1 << 13)
     table = sa.sideaware_torch_side_index().cpu().numpy()
     assert table.shape == (info["num_sms"],)
-    xcd = table & 7
-    counts = np.bincount(xcd, minlength=lib.sideaware_num_xcds())
-    assert counts.sum() == info["num_sms"] and counts[0] == info["side0"]
-    # ranks within each XCD count up from zero without gaps
-    for x in range(lib.sideaware_num_xcds()):
-        ranks = np.sort(table[xcd == x] >> 3)
-        assert np.array_equal(ranks, np.arange(len(ranks)) & 0x1f)
+    side = table & 1
+    counts = np.bincount(side, minlength=2)
+    assert counts.sum() == info["num_sms"] and counts[0] == info["side0"] and counts[1] == info["side1"]
+    assert info["min"] == min(info["side0"], info["side1"]) or lib.sideaware_num_xcds() == 1
+    if lib.sideaware_num_xcds() == 8:
+        assert info["side0"] == info["side1"] == info["num_sms"] // 2
+    # ranks within each side count up from zero without gaps (the reference's table layout)
+    for sd in range(2):
+        ranks = np.sort(table[side == sd] >> 1)
+        assert np.array_equal(ranks, np.arange(len(ranks)) & 0x7f)
     # the host copy the library returns a pointer to holds the same bytes
     host = (ctypes.c_ubyte * info["num_sms"]).from_address(sa.sideaware_cpu_side_index())
     assert np.array_equal(np.frombuffer(host, dtype=np.uint8), table)

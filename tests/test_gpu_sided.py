@@ -207,3 +207,40 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
     torch.cuda.synchronize()
     assert counts(lib)[0] == before[0] + 1
     assert torch.equal(y, x.float() * 2.0 + b)
+
+
+M64 = (1 << 64) - 1
+
+
+def splitmix64(x):
+    z = (x * 0x9e3779b97f4a7c15 + 0x9e3779b97f4a7c15) & M64
+    z = ((z ^ (z >> 30)) * 0xbf58476d1ce4e5b9) & M64
+    z = ((z ^ (z >> 27)) * 0x94d049bb133111eb) & M64
+    return z ^ (z >> 31)
+
+
+def test_probe_sides_measures_what_the_arena_probe_measured(sa, lib):
+    """sideaware_probe_sides times loads at seeded sample granules of any device memory; on the
+    pool's own memory its answers must be those of sideaware_side_of (measured once, when the arena
+    was acquired), wherever the timing was decisive."""
+    stream = torch.cuda.current_stream().cuda_stream
+    region = torch.empty(320 * MiB, dtype=torch.uint8, device="cuda")
+    count, seed, nbytes = 300, 5, 320 * MiB
+    sides = torch.full((count + 4,), 9, dtype=torch.int32, device="cuda")
+    assert lib.sideaware_probe_sides(region.data_ptr(), nbytes, seed, count, sides.data_ptr(), 0, stream) == 0
+    torch.cuda.synchronize()
+    got = sides.cpu().tolist()
+    assert got[count:] == [9] * 4
+    decisive = 0
+    for i in range(count):
+        offset = (splitmix64((seed + i) & M64) % (nbytes // 8192)) * 8192
+        want = lib.sideaware_side_of(region.data_ptr() + offset)
+        assert want in (0, 1) and got[i] in (-1, want), (i, offset, got[i], want)
+        decisive += got[i] >= 0
+    assert decisive >= 0.9 * count
+    # bad arguments are refused with a message, nothing is launched
+    assert lib.sideaware_probe_sides(region.data_ptr(), 64 * MiB, 1, 8, sides.data_ptr(), 0, stream) != 0
+    assert b"128 MiB" in lib.sideaware_last_error()
+    assert lib.sideaware_probe_sides(region.data_ptr() + 16, nbytes - 8192, 1, 8, sides.data_ptr(), 0, stream) != 0
+    assert lib.sideaware_probe_sides(region.data_ptr(), nbytes, 1, 0, sides.data_ptr(), 0, stream) != 0
+    lib.sideaware_clear_error()
