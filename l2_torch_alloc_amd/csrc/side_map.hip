@@ -355,9 +355,11 @@ void SideRegistry::add_arena(void* base, size_t bytes) {
     a.base = (uintptr_t)base;
     a.bytes = bytes;
     if (hash_.known && bytes >= (1u << kSidePairLog2) && a.base % (1u << kSidePairLog2) == 0) {
-        // The arena's constant: a vote over granules spread across it.  One sample that
-        // contradicts the others means the arena is not laid out as the hash says.
-        constexpr int kSamples = 48;
+        // The arena's constant: a vote over granules spread across it.  A few samples may go the
+        // other way (a timing that went wrong, or a stretch of the arena that is not physically
+        // contiguous with the rest: there the sided map is simply wrong, which costs speed, not
+        // results); more than a few mean the arena is not laid out as the hash says.
+        constexpr int kSamples = 192;
         std::vector<uint64_t> offsets;
         uint64_t lcg = 0x2545f4914f6cdd1dull ^ (uint64_t)a.base;
         const uint64_t granules = bytes >> kSideGranuleLog2;
@@ -376,9 +378,10 @@ void SideRegistry::add_arena(void* base, size_t bytes) {
             }
             const int valid = votes[0] + votes[1];
             if (side_debug()) std::fprintf(stderr, "sideaware: arena %p (%zu MiB): votes %d / %d\n", base, bytes >> 20, votes[0], votes[1]);
-            if (valid >= kSamples * 3 / 4 && (votes[0] == 0 || votes[1] == 0)) {
+            const int minority = votes[0] < votes[1] ? votes[0] : votes[1];
+            if (valid >= kSamples * 3 / 4 && minority * 32 <= valid) {
                 a.known = true;
-                a.flip = votes[1] ? 1u : 0u;
+                a.flip = votes[1] > votes[0] ? 1u : 0u;
             }
         }
     }

