@@ -166,6 +166,14 @@ int sideaware_xcd_dealing_verified(void);
  * Returns 0, or a HIP error code after recording a message for sideaware_last_error. */
 int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
                           int device, sideaware_stream_t stream);
+/* The same measurement for callers that cannot allocate (code under stream capture, tight serving
+ * loops, harnesses that forbid it): no counterpart in the reference.  It allocates nothing and
+ * frees nothing; its work space is a static device array of 32 KiB that every device the library
+ * runs on holds until the process ends, so `count` may be at most 512 (more is refused with an
+ * error), and two calls that overlap on one device race on that array: give them one stream, or
+ * order them yourself.  Same results as sideaware_probe_sides. */
+int sideaware_probe_sides_noalloc(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
+                                  int device, sideaware_stream_t stream);
 unsigned long long sideaware_side_address_mask(void);
 int sideaware_side_of(const void* ptr);
 int sideaware_stream_dealing(sideaware_stream_t stream);

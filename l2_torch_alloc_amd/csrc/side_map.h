@@ -113,8 +113,14 @@ public:
 
     // Times loads from every XCD at `count` sample granules of [region, region + bytes) on
     // `stream` and writes, for each, the side that is clearly nearer (0 or 1), or -1, to the device
-    // array `sides`.  Returns 0, or a negative code for a bad argument (-1) or no memory (-4).
-    int probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream);
+    // array `sides`.  With allocate == false nothing is allocated: the work space is a static
+    // device array (init_static_scratch must have run), count is at most kNoAllocMaxSamples, and
+    // calls that overlap on one device share (and race on) that array.  Returns 0, or a negative
+    // code for a bad argument (-1), too many samples (-2), no static array (-3), no memory (-4).
+    int probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream,
+                    bool allocate);
+    void init_static_scratch();
+    static constexpr int kNoAllocMaxSamples = 512;
 
     // For tests and tools: forget what was measured / pretend.
     void set_hash_for_test(const SideHash& h) { std::lock_guard<std::mutex> g(mu_); hash_ = h; discovered_ = true; }
@@ -141,6 +147,7 @@ private:
     uint64_t* probe_offsets_ = nullptr;        // device
     unsigned int* probe_lat_ = nullptr;        // device
     volatile unsigned int* feedback_ = nullptr;     // pinned host, kFeedbackSlots * 16 words
+    unsigned int* static_scratch_ = nullptr;        // this device's address of the static work array
     std::unordered_map<void*, int> slot_of_stream_;
     static constexpr int kFeedbackSlots = 64;
     static constexpr int kMaxProbe = 512;

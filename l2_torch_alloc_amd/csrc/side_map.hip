@@ -164,7 +164,23 @@ bool side_probing_enabled() {
 
 }  // namespace
 
-// The probe behind sideaware_probe_sides: everything runs on the
+// The allocation-free probe's scratch: the per-XCD times of up to kNoAllocMaxSamples samples plus
+// the scrub kernel's sink.  One copy per device the library runs on, held until the process ends.
+static __device__ __align__(256) unsigned int scratch[16 * SideRegistry::kNoAllocMaxSamples + 64];
+
+void SideRegistry::init_static_scratch() {
+    std::lock_guard<std::mutex> g(mu_);
+    if (static_scratch_) return;
+    DeviceGuard dev(device_);
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    static_scratch_ = (unsigned int*)ptr;            // this device's copy of the array
+}
+
+// The probe behind sideaware_probe_sides and sideaware_probe_sides_noalloc: everything runs on the
 // caller's stream, the results stay on the device.  `work` holds 16 * count + 16 words.
 int SideRegistry::probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides,
                                   void* stream, unsigned int* work) {
@@ -187,8 +203,19 @@ int SideRegistry::probe_on_stream(const void* region, size_t bytes, unsigned lon
 }
 
 int SideRegistry::probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides,
-                              void* stream) {
+                              void* stream, bool allocate) {
     if (!region || !sides || count < 1 || bytes < kScrubBytes || ((uintptr_t)region & ((1u << kSideGranuleLog2) - 1))) return -1;
+    if (!allocate) {
+        // no allocation of any kind: the device's static array is the work space
+        if (count > kNoAllocMaxSamples) return -2;
+        unsigned int* work;
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            work = static_scratch_;
+        }
+        if (!work) return -3;
+        return probe_on_stream(region, bytes, seed, count, sides, stream, work);
+    }
     DeviceGuard dev(device_);
     hipStream_t st = (hipStream_t)stream;
     unsigned int* work = nullptr;

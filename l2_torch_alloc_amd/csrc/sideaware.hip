@@ -331,6 +331,7 @@ void DeviceContext::initialize() {
 
     backing = std::make_unique<HipBacking>(device);
     backing->sides().discover();                 // which address bits decide the half of the device (a few ms)
+    backing->sides().init_static_scratch();      // this device's address of the allocation-free probe's work array
     side_summary[4] = side_hash_mask(this);
     pool = std::make_unique<Pool>(backing.get());
     // The reference trims its cache from 16 GiB down to 2 GiB on an 80 GB part
@@ -1176,23 +1177,31 @@ int sideaware_stream_dealing(sideaware_stream_t stream) {
     return c->backing->sides().feedback_slot(stream, &dealing) ? (int)dealing : -1;
 }
 
-int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
-                          int device, sideaware_stream_t stream) {
+static int probe_sides_common(const char* what, const void* region, size_t num_bytes, unsigned long long seed, int count,
+                              int* sides, int device, sideaware_stream_t stream, bool allocate) {
     DeviceContext* c = get_context(device);
     if (!c) return (int)hipErrorNoDevice;
-    const int rc = c->backing->sides().probe_sides(region, num_bytes, seed, count, sides, stream);
-    if (rc == 0) return 0;
-    if (rc == -1) {
-        set_error("probe_sides: region (%p, granule-aligned), sides (%p), count (%d, at least 1) or num_bytes (%zu, at least "
-                  "128 MiB) is not acceptable", region, (void*)sides, count, num_bytes);
-        return (int)hipErrorInvalidValue;
+    const int rc = c->backing->sides().probe_sides(region, num_bytes, seed, count, sides, stream, allocate);
+    switch (rc) {
+        case 0: return 0;
+        case -1: set_error("%s: region (%p, granule-aligned), sides (%p), count (%d, at least 1) or num_bytes (%zu, at least "
+                           "128 MiB) is not acceptable", what, region, (void*)sides, count, num_bytes); return (int)hipErrorInvalidValue;
+        case -2: set_error("%s: %d samples asked for, the static work array holds %d", what, count,
+                           SideRegistry::kNoAllocMaxSamples); return (int)hipErrorInvalidValue;
+        case -3: set_error("%s: the static work array's device address is not known", what); return (int)hipErrorNotInitialized;
+        case -4: set_error("%s: no memory for the work space", what); return (int)hipErrorOutOfMemory;
+        default: set_error("%s: launch failed: %s", what, hipGetErrorString((hipError_t)rc)); return rc;
     }
-    if (rc == -4) {
-        set_error("probe_sides: no memory for the work space");
-        return (int)hipErrorOutOfMemory;
-    }
-    set_error("probe_sides: launch failed: %s", hipGetErrorString((hipError_t)rc));
-    return rc;
+}
+
+int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
+                          int device, sideaware_stream_t stream) {
+    return probe_sides_common("probe_sides", region, num_bytes, seed, count, sides, device, stream, /*allocate=*/true);
+}
+
+int sideaware_probe_sides_noalloc(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
+                                  int device, sideaware_stream_t stream) {
+    return probe_sides_common("probe_sides_noalloc", region, num_bytes, seed, count, sides, device, stream, /*allocate=*/false);
 }
 
 void sideaware_launch_counts(unsigned long long* sided, unsigned long long* striped) {
