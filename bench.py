@@ -574,36 +574,32 @@ def bench_churn_raw_calls(n_ops=10000, live_cap=64 * GiB):
     from l2_torch_alloc_amd import wrapper
     lib = wrapper.library()
     sizes = churn_sizes(n_ops)
-    lib.sideaware_oom_raises(0)                  # a null from a ctypes call is checked here, not thrown
     before = wrapper.sideaware_alloc_stats()
     live, live_bytes = [], 0
     t_alloc, t_free = [], []
-    try:
-        for size in sizes:
+    for size in sizes:
+        t0 = time.perf_counter_ns()
+        x = lib.sideaware_malloc_auto(size, 0, None)
+        t1 = time.perf_counter_ns()
+        y = lib.sideaware_malloc_auto(size, 0, None)
+        t2 = time.perf_counter_ns()
+        if not x or not y:
+            raise RuntimeError("the pool returned null for %d bytes" % size)
+        t_alloc.append(t1 - t0)
+        t_alloc.append(t2 - t1)
+        t0 = time.perf_counter_ns()
+        lib.sideaware_free_auto(y, size, 0, None)
+        t_free.append(time.perf_counter_ns() - t0)
+        live.append((x, size))
+        live_bytes += size
+        while live_bytes > live_cap:
+            old, old_size = live.pop(0)
+            live_bytes -= old_size
             t0 = time.perf_counter_ns()
-            x = lib.sideaware_malloc_auto(size, 0, None)
-            t1 = time.perf_counter_ns()
-            y = lib.sideaware_malloc_auto(size, 0, None)
-            t2 = time.perf_counter_ns()
-            if not x or not y:
-                raise RuntimeError("the pool returned null for %d bytes" % size)
-            t_alloc.append(t1 - t0)
-            t_alloc.append(t2 - t1)
-            t0 = time.perf_counter_ns()
-            lib.sideaware_free_auto(y, size, 0, None)
-            t_free.append(time.perf_counter_ns() - t0)
-            live.append((x, size))
-            live_bytes += size
-            while live_bytes > live_cap:
-                old, old_size = live.pop(0)
-                live_bytes -= old_size
-                t0 = time.perf_counter_ns()
-                lib.sideaware_free_auto(old, old_size, 0, None)
-                t_free.append(time.perf_counter_ns() - t0)
-        for old, old_size in live:
             lib.sideaware_free_auto(old, old_size, 0, None)
-    finally:
-        lib.sideaware_oom_raises(1)
+            t_free.append(time.perf_counter_ns() - t0)
+    for old, old_size in live:
+        lib.sideaware_free_auto(old, old_size, 0, None)
     after = wrapper.sideaware_alloc_stats()
 
     def pct(v, p):
@@ -623,7 +619,6 @@ def bench_raw_alloc_calls(n=20000):
     from l2_torch_alloc_amd import wrapper
     lib = wrapper.library()
     out = {}
-    lib.sideaware_oom_raises(0)                  # nulls are not expected here, and must not become C++ exceptions
     for label, size in (("small_64KiB", 64 * 1024), ("large_64MiB", 64 * MiB)):
         p = lib.sideaware_malloc_auto(size, 0, None)
         lib.sideaware_free_auto(p, size, 0, None)
@@ -640,7 +635,6 @@ def bench_raw_alloc_calls(n=20000):
         tf.sort()
         out[label] = {"alloc_p50_us": ta[n // 2] / 1e3, "alloc_p99_us": ta[int(n * 0.99)] / 1e3,
                       "free_p50_us": tf[n // 2] / 1e3, "free_p99_us": tf[int(n * 0.99)] / 1e3}
-    lib.sideaware_oom_raises(1)
     return out
 
 

@@ -1,4 +1,4 @@
-// hbm_ceiling.so: framework-free streaming kernels for gfx950 that measure what the memory system of
+// bench_ceiling_kernels.so: framework-free streaming kernels for gfx950 that measure what the memory system of
 // an MI355X delivers to the simplest possible read, write and copy loops.  They share nothing with
 // the elementwise template (no op hooks, no launch planner): `bench.py --ceiling` times them beside
 // the library's own kernels so that "the hardware tops out here" is a measurement, not a claim.
@@ -18,7 +18,7 @@ enum : int {
     kLaneContiguous = 4,   // a lane takes K consecutive vectors instead of K vectors a block apart
     kWaitStores = 8,       // persistent kernels: stores are acknowledged before the next loads are issued
     kPrefetch = 16,        // persistent copies: the next chunk's loads are issued before this chunk's stores
-    kSplitRoles = 16,      // tile kernel: workgroup pairs alternate between reading src and filling dst
+    kSplitRoles = 32,      // tile kernel: workgroup pairs alternate between reading src and filling dst
 };
 
 template <bool NT>
@@ -372,6 +372,7 @@ int hbm_ceiling_tile(void* dst, const void* src, size_t bytes, int k, int block,
     if (block < 64 || block > 1024 || (block & (block - 1))) return fail("block must be a power of two in 64..1024");
     if (stripe_log2 < 0 || stripe_log2 > 12) return fail("stripe_log2 must be in 0..12");
     if (!dst && !src) return fail("nothing to do");
+    if ((flags & kSplitRoles) && (!dst || !src)) return fail("split roles needs both buffers");
     if (!sink) return fail("sink must point at four bytes of device memory");
     const size_t tile_bytes = (size_t)k * block * 16;
     const size_t period = (tile_bytes * 8) << stripe_log2;

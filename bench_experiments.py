@@ -172,16 +172,37 @@ def inflight_ab(steps):
 
 # ------------------------------------------------------------------------------------- ceilings
 
-NT_LOADS, NT_STORES, LANE_CONTIGUOUS, WAIT_STORES, SPLIT_ROLES = 1, 2, 4, 8, 16
+NT_LOADS, NT_STORES, LANE_CONTIGUOUS, WAIT_STORES, PREFETCH, SPLIT_ROLES = 1, 2, 4, 8, 16, 32
+
+
+CEILING_SOURCE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_ceiling_kernels.hip")
+CEILING_LIBRARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_ceiling_kernels.so")
+
+
+def build_ceiling_library(force=False):
+    """Compiles the framework-free streaming kernels (bench_ceiling_kernels.hip) for gfx950 with
+    hipcc, in-tree, when the built file is missing or older than its source."""
+    import shutil
+    import subprocess
+    if not force and os.path.exists(CEILING_LIBRARY) and os.path.getmtime(CEILING_LIBRARY) >= os.path.getmtime(CEILING_SOURCE):
+        return CEILING_LIBRARY
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-fvisibility=hidden",
+           CEILING_SOURCE, "-o", CEILING_LIBRARY + ".tmp"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + proc.stderr)
+    os.replace(CEILING_LIBRARY + ".tmp", CEILING_LIBRARY)
+    return CEILING_LIBRARY
 
 
 def ceiling_library():
-    """The framework-free streaming kernels (csrc/hbm_ceiling.hip), bound with ctypes."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "l2_torch_alloc_amd", "hbm_ceiling.so")
-    if not os.path.exists(path):
-        raise FileNotFoundError("%s is not built; run `python -m l2_torch_alloc_amd.build`" % path)
+    """The framework-free streaming kernels (bench_ceiling_kernels.hip), built on demand and bound
+    with ctypes: measurement support for `bench.py --ceiling`, no part of the library."""
+    path = build_ceiling_library()
     lib = ctypes.CDLL(path)
-    vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
     lib.hbm_ceiling_tile.argtypes = [vp, vp, sz, ci, ci, ci, ci, vp, vp, vp]
     lib.hbm_ceiling_tile.restype = ci
     lib.hbm_ceiling_policy.argtypes = [vp, vp, sz, ci, ctypes.c_char_p, ctypes.c_char_p, ci, vp, vp]

@@ -135,6 +135,12 @@ void sideaware_reserve_limit(size_t bytes);
  * becomes a tensor whose data pointer is 0), and the exception reaches Python as a RuntimeError.
  * Only sideaware_malloc_auto is affected; the entry points that return an error code keep doing so. */
 void sideaware_oom_raises(int enable);
+/* sideaware_malloc_auto for C++ hosts that do not check the pointer: the entry point to name in
+ * torch.cuda.memory.CUDAPluggableAllocator.  Where sideaware_malloc_auto would return null for a
+ * non-zero size it raises a C++ std::runtime_error ("sideaware: out of memory: ..."), whatever
+ * sideaware_oom_raises says.  It is the only entry point that throws unconditionally; never call it
+ * through C frames (ctypes is C). */
+void* sideaware_malloc_auto_raising(size_t size, int device, sideaware_stream_t stream);
 /* Size of the arenas that large regions are carved from (default 4 GiB); 0 gives every large
  * region a driver allocation of its own, as in the reference. */
 void sideaware_arena_bytes(size_t bytes);

@@ -80,25 +80,5 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
     return LIB_PATH
 
 
-CEILING_LIB_PATH = os.path.join(PKG_DIR, "hbm_ceiling.so")
-
-
-def build_ceiling_library(force: bool = True) -> str:
-    """Compiles the framework-free streaming kernels that ``bench.py --ceiling`` times beside the
-    library's own (csrc/hbm_ceiling.hip): measurement support, not part of the product path."""
-    src = os.path.join(CSRC, "hbm_ceiling.hip")
-    if not force and os.path.exists(CEILING_LIB_PATH) and os.path.getmtime(CEILING_LIB_PATH) >= os.path.getmtime(src):
-        return CEILING_LIB_PATH
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-fvisibility=hidden",
-           src, "-o", CEILING_LIB_PATH + ".tmp"]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + proc.stderr)
-    os.replace(CEILING_LIB_PATH + ".tmp", CEILING_LIB_PATH)
-    return CEILING_LIB_PATH
-
-
 if __name__ == "__main__":
     print(build_library(force=True, verbose=True))
-    print(build_ceiling_library(force=True))

@@ -74,11 +74,11 @@ void HipBacking::release(void* ptr, size_t) {
 // Where in the free run [lo, hi) a block of `bytes` should start so that its granules alternate
 // between the device's halves the same way every other block's do; 0 when nothing is known about
 // the arena the run lies in.
-uintptr_t HipBacking::place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) {
+uintptr_t HipBacking::place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes, bool lines) {
     uintptr_t base = 0;
     unsigned int flip = 0;
     if (!sides_.arena_of((const void*)lo, &base, &flip)) return 0;
-    return canonical_start(sides_.hash(), flip, base, lo, hi, bytes);
+    return canonical_start(sides_.hash(), flip, base, lo, hi, bytes, lines);
 }
 
 void HipBacking::sync_device() {

@@ -17,7 +17,7 @@ public:
     void sync_device() override;
     void order_after(void* producer, void* consumer) override;
     int free_foreign(void* ptr, void* stream) override;
-    uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) override;
+    uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes, bool lines) override;
 
     // What was measured about the arenas handed to the pool (side_map.h).
     SideRegistry& sides() { return sides_; }

@@ -115,24 +115,27 @@ void Pool::extent_insert_locked(int kind, uintptr_t addr, Extent e) {
 // block is the extent's front.  With `canonical` the backing store is asked where in the extent the
 // block should start so that the device's memory halves alternate through it like through every
 // other block placed this way (Backing::place_canonical); the first few extents in best-fit order
-// are tried, and when none can hold such a block (or the backing store knows no rule) the front of
-// the best fit is taken after all.
+// are tried, and when none can hold such a block without a large hole in front of it (or the
+// backing store knows no rule) the front of the best fit is taken after all.
 bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* taken, bool canonical) {
     ExtentIndex& ix = free_[kind];
     auto sit = ix.by_size.lower_bound({bytes, 0});
     if (sit == ix.by_size.end()) return false;
     uintptr_t start = sit->second;
     if (canonical) {
+        bool placed = false;
         int tries = 0;
         for (auto cand = sit; cand != ix.by_size.end() && tries < kCanonicalTries; ++cand, ++tries) {
-            const uintptr_t at = backing_->place_canonical(cand->second, cand->second + cand->first, bytes);
+            const uintptr_t at = backing_->place_canonical(cand->second, cand->second + cand->first, bytes, /*lines=*/true);
             if (at == 0) continue;
             assert(at >= cand->second && at + bytes <= cand->second + cand->first && at % kRegionAlign == 0);
+            if (at - cand->second > std::max<size_t>(kCanonicalSlack, bytes / kCanonicalGapDivisor)) continue;   // too large a hole in front
             sit = cand;
             start = at;
-            st_.canonical_placements++;
+            placed = true;
             break;
         }
+        if (placed) st_.canonical_placements++;
     }
     const uintptr_t ext_addr = sit->second;
     auto ait = ix.by_addr.find(ext_addr);

@@ -781,19 +781,28 @@ extern "C" {
 
 // ---- allocation -------------------------------------------------------------------------------
 
+// PyTorch's pluggable-allocator shim does not look at the pointer it gets: a null would become a
+// tensor whose data pointer is 0, and the first kernel on it a GPU fault.  Its frames are C++, so an
+// exception thrown through them arrives in Python as a RuntimeError.
+static void* raise_out_of_memory(size_t size, int device) {
+    char msg[256];
+    std::snprintf(msg, sizeof msg, "sideaware: out of memory: tried to allocate %zu bytes on device %d "
+                  "(see sideaware_alloc_stats)", size, device);
+    set_error("%s", msg);
+    throw std::runtime_error(msg);
+}
+
 void* sideaware_malloc_auto(size_t size, int device, sideaware_stream_t stream) {
     DeviceContext* ctx = get_context(device);
     void* p = ctx ? ctx->pool->allocate(size, stream, /*always_large=*/false) : nullptr;
-    if (!p && size != 0 && g_oom_raises.load(std::memory_order_relaxed)) {
-        // PyTorch's pluggable-allocator shim does not look at the pointer it gets: a null would
-        // become a tensor whose data pointer is 0, and the first kernel on it a GPU fault.  Its
-        // frames are C++, so an exception thrown here arrives in Python as a RuntimeError.
-        char msg[256];
-        std::snprintf(msg, sizeof msg, "sideaware: out of memory: tried to allocate %zu bytes on device %d "
-                      "(see sideaware_alloc_stats)", size, device);
-        set_error("%s", msg);
-        throw std::runtime_error(msg);
-    }
+    if (!p && size != 0 && g_oom_raises.load(std::memory_order_relaxed)) return raise_out_of_memory(size, device);
+    return p;
+}
+
+void* sideaware_malloc_auto_raising(size_t size, int device, sideaware_stream_t stream) {
+    DeviceContext* ctx = get_context(device);
+    void* p = ctx ? ctx->pool->allocate(size, stream, /*always_large=*/false) : nullptr;
+    if (!p && size != 0) return raise_out_of_memory(size, device);
     return p;
 }
 

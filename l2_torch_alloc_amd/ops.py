@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -17,12 +18,28 @@ import torch
 from . import headers, wrapper
 
 _kernel_ids: Dict[Tuple, int] = {}
+_CHECK_POSITION_VALUES = os.environ.get("SIDEAWARE_CHECK_POSITIONS") == "1"
+
+_HEADER_BUILDERS = {
+    "rope": headers.rope_header,
+    "rope_half": headers.rope_half_header,
+    "scale_bias_bf16": headers.scale_bias_bf16_header,
+    "mxfp8_quantize": headers.mxfp8_quantize_header,
+    "mxfp8_dequantize": headers.mxfp8_dequantize_header,
+    "fill": headers.fill_header,
+}
 
 
-def _kernel(key: Tuple, make_header) -> int:
+@torch.compiler.assume_constant_result
+def _kernel(builder: str, args: Tuple = (), kwargs: Tuple = ()) -> int:
+    """The kernel id of the op whose header is ``_HEADER_BUILDERS[builder](*args, **dict(kwargs))``,
+    registering it on first use.  Everything it takes is a constant (strings, ints, bools), so a
+    tracer evaluates the call once, while it traces, and keeps the id as a constant of the graph:
+    an op whose first use falls inside ``torch.compile(fullgraph=True)`` needs no eager warm-up."""
+    key = (builder, args, kwargs)
     kid = _kernel_ids.get(key)
     if kid is None:
-        kid = wrapper.sideaware_create_kernel(make_header())
+        kid = wrapper.sideaware_create_kernel(_HEADER_BUILDERS[builder](*args, **dict(kwargs)))
         _kernel_ids[key] = kid
     return kid
 
@@ -61,10 +78,17 @@ def freqs_cis_table(head_dim: int, end: int, theta: float, use_scaled: bool = Fa
 _ROPE_DTYPES = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
 
 
-def _check_positions(positions: torch.Tensor, tokens: int) -> None:
+def _check_positions(positions: torch.Tensor, tokens: int, x: torch.Tensor, rows: int) -> None:
+    """The kernel reads table row ``positions[token]`` without a bound (a check per element would
+    cost more than the op): shape, type and device are checked here, and with
+    ``SIDEAWARE_CHECK_POSITIONS=1`` in the environment the values too (a device round trip)."""
     assert positions.dtype == torch.int32 and positions.is_cuda and positions.is_contiguous(), \
         "positions are a contiguous int32 device tensor"
+    assert positions.device == x.device, "positions live on the activations' device"
     assert positions.numel() == tokens, "one position per token of the flattened (B, T) axes"
+    if _CHECK_POSITION_VALUES and tokens:
+        lo, hi = int(positions.min()), int(positions.max())
+        assert 0 <= lo and hi < rows, "positions must lie in [0, %d): got %d .. %d" % (rows, lo, hi)
 
 
 def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q: int, n_kv: int,
@@ -83,7 +107,7 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
     else:
         assert layout == "heads", "positions go with separate q / k tensors"
         assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
-        _check_positions(positions, B * T)
+        _check_positions(positions, B * T, x, freqs.shape[0])
         T = 0                                   # the sequence length is not part of the compiled text
     if out is None:
         out = x
@@ -93,11 +117,8 @@ def _rope(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor], n_q
             # value heads are skipped by the kernel (neither read nor written): out of place they
             # have to be carried over by a copy first
             torch.ops.sideaware.memcpy(out, x)
-    key = (T, n_q, n_kv, head_dim, dtype, layout, backward, positions is not None)
-    kid = _kernel_ids.get(key)
-    if kid is None:
-        kid = _kernel(key, lambda: headers.rope_header(max(T, 1), n_q, n_kv, head_dim, dtype, layout, backward,
-                                                       positions=positions is not None))
+    kid = _kernel("rope", (max(T, 1), n_q, n_kv, head_dim, dtype, layout, backward),
+                  (("positions", positions is not None),))
     _elementwise(kid, out, None, None, None, x, freqs, None, None, positions, 0, 0, 0)
     return out
 
@@ -159,8 +180,7 @@ def _rope_heads_many(tensors, freqs: torch.Tensor, backward: bool, positions: Op
     assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
     for t in tensors:
         assert t.dim() == 4 and t.shape[1] == T and t.shape[3] == head_dim and t.dtype == first.dtype
-    key = ("rope_heads_at_launch", T, head_dim, dtype, backward)
-    kid = _kernel(key, lambda: headers.rope_header(T, 0, 0, head_dim, dtype, "heads", backward, heads_at_launch=True))
+    kid = _kernel("rope", (T, 0, 0, head_dim, dtype, "heads", backward), (("heads_at_launch", True),))
     elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], None, t.shape[2]) for t in tensors])
     return tensors
 
@@ -172,16 +192,15 @@ def _rope_many_at_positions(tensors, freqs, backward: bool, positions: torch.Ten
     if dtype is None:
         raise TypeError("RoPE storage is float32, bfloat16 or float16")
     assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
-    _check_positions(positions, B * T)
+    _check_positions(positions, B * T, first, freqs.shape[0])
     for t in tensors:
         assert t.dim() == 4 and t.is_contiguous() and t.shape[:2] == first.shape[:2] and t.shape[3] == head_dim \
             and t.dtype == first.dtype
-    key = ("rope_many_at_positions", head_dim, dtype, backward, half)
+    launch_time = (("heads_at_launch", True), ("positions", True))
     if half:
-        make = lambda: headers.rope_half_header(1, 0, head_dim, dtype, backward, heads_at_launch=True, positions=True)
+        kid = _kernel("rope_half", (1, 0, head_dim, dtype, backward), launch_time)
     else:
-        make = lambda: headers.rope_header(1, 0, 0, head_dim, dtype, "heads", backward, heads_at_launch=True, positions=True)
-    kid = _kernel(key, make)
+        kid = _kernel("rope", (1, 0, 0, head_dim, dtype, "heads", backward), launch_time)
     elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], positions, t.shape[2]) for t in tensors])
     return tensors
 
@@ -212,14 +231,12 @@ def _rope_half(x: torch.Tensor, freqs: torch.Tensor, out: Optional[torch.Tensor]
     else:
         assert not heads_first, "positions are per token of a (B, T, heads, head_dim) tensor"
         assert freqs.dtype == torch.float32 and freqs.dim() == 2 and freqs.shape[1] == head_dim
-        _check_positions(positions, x.shape[0] * T)
+        _check_positions(positions, x.shape[0] * T, x, freqs.shape[0])
         T = 1                                   # the sequence length is not part of the compiled text
     if out is None:
         out = x
     assert out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()
-    key = ("rope_half", T, heads, head_dim, dtype, heads_first, backward, positions is not None)
-    kid = _kernel(key, lambda: headers.rope_half_header(T, heads, head_dim, dtype, backward, heads_first,
-                                                        positions=positions is not None))
+    kid = _kernel("rope_half", (T, heads, head_dim, dtype, backward, heads_first), (("positions", positions is not None),))
     _elementwise(kid, out, None, None, None, x, freqs, None, None, positions, 0, 0, 0)
     return out
 
@@ -251,8 +268,7 @@ def rope_half_forward_many(tensors, freqs, backward: bool = False, positions=Non
     assert freqs.dtype == torch.float32 and tuple(freqs.shape) == (T, head_dim)
     for t in tensors:
         assert t.dim() == 4 and t.is_contiguous() and t.shape[1] == T and t.shape[3] == head_dim and t.dtype == first.dtype
-    key = ("rope_half_heads_at_launch", T, head_dim, dtype, backward)
-    kid = _kernel(key, lambda: headers.rope_half_header(T, 0, head_dim, dtype, backward, heads_at_launch=True))
+    kid = _kernel("rope_half", (T, 0, head_dim, dtype, backward), (("heads_at_launch", True),))
     elementwise_batch(kid, [(t.numel() * t.element_size(), [t], [t, freqs], None, t.shape[2]) for t in tensors])
     return tensors
 
@@ -263,7 +279,7 @@ def scale_bias_bf16(x: torch.Tensor, scale_bias: torch.Tensor, out: Optional[tor
     assert x.dtype == torch.bfloat16 and scale_bias.dtype == torch.float32 and scale_bias.numel() >= 2
     if out is None:
         out = torch.empty_like(x)
-    kid = _kernel(("scale_bias_bf16",), headers.scale_bias_bf16_header)
+    kid = _kernel("scale_bias_bf16")
     _elementwise(kid, out, None, None, None, x, None, None, None, scale_bias, 0, 0, 0)
     return out
 
@@ -277,7 +293,7 @@ def mxfp8_quantize(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Op
     if scales is None:
         scales = torch.empty(x.numel() // 32, dtype=torch.uint8, device=x.device)
     assert q.dtype == torch.uint8 and q.numel() == x.numel() and scales.numel() == x.numel() // 32
-    kid = _kernel(("mxfp8_quantize",), headers.mxfp8_quantize_header)
+    kid = _kernel("mxfp8_quantize")
     device, stream = wrapper._device_and_stream()
     # num_bytes is the byte length of the wider array, the bf16 input, which the custom-op wrapper
     # cannot know (it sizes the launch from out0, as the reference's does): call the C entry point.
@@ -295,7 +311,7 @@ def mxfp8_dequantize(q: torch.Tensor, scales: torch.Tensor, out: Optional[torch.
     if out is None:
         out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
     assert out.dtype == torch.bfloat16 and out.numel() == q.numel()
-    kid = _kernel(("mxfp8_dequantize",), headers.mxfp8_dequantize_header)
+    kid = _kernel("mxfp8_dequantize")
     # out0 is the wider array, so the custom op's own sizing (from out0) is the right one
     _elementwise(kid, out, None, None, None, q, None, None, None, scales, 0, 0, 0)
     return out
@@ -303,6 +319,6 @@ def mxfp8_dequantize(q: torch.Tensor, scales: torch.Tensor, out: Optional[torch.
 
 def fill_int32(out: torch.Tensor, value: int):
     """Writes a 32-bit pattern over ``out`` (byte size a multiple of 16): an output-only op."""
-    kid = _kernel(("fill",), headers.fill_header)
+    kid = _kernel("fill")
     _elementwise(kid, out, None, None, None, None, None, None, None, None, int(value), 0, 0)
     return out

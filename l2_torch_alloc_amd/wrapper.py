@@ -39,6 +39,7 @@ _vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 # travel in the same integer register on x86-64, so either declaration works.
 _SIGNATURES = {
     "sideaware_malloc_auto": (_vp, [_sz, _ci, _vp]),
+    "sideaware_malloc_auto_raising": (_vp, [_sz, _ci, _vp]),
     "sideaware_free_auto": (None, [_vp, _sz, _ci, _vp]),
     "sideaware_malloc": (_ci, [ctypes.POINTER(_vp), _sz]),
     "sideaware_free": (_ci, [_vp]),
@@ -178,14 +179,14 @@ def sideaware_init(path: str = DEFAULT_LIBRARY, install_allocator: bool = True) 
         raise RuntimeError("sideaware needs a GPU: torch.cuda.is_available() is False")
     path = os.path.abspath(path)
     if install_allocator and not _allocator_installed:
-        allocator = torch.cuda.memory.CUDAPluggableAllocator(path, "sideaware_malloc_auto", "sideaware_free_auto")
+        # PyTorch does not check the pointer its pluggable allocator returns: it gets the entry point
+        # that raises (a RuntimeError in Python) when the pool is exhausted instead of returning null.
+        # sideaware_malloc_auto itself keeps the reference's contract (null), for ctypes callers.
+        allocator = torch.cuda.memory.CUDAPluggableAllocator(path, "sideaware_malloc_auto_raising", "sideaware_free_auto")
         torch.cuda.memory.change_current_allocator(allocator)
         _allocator_installed = True
     if _lib is None:
         _lib = bind(path)
-    # PyTorch does not check the pointer its pluggable allocator returns: have an exhausted pool
-    # raise (a RuntimeError in Python) instead of handing PyTorch a null
-    _lib.sideaware_oom_raises(1)
     _register_ops()
     _refresh_metadata()
     # the reference prints this line when initialisation is done (example_wrapper.py:109); here it

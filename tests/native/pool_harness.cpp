@@ -70,13 +70,13 @@ struct FakeBacking final : Backing {
         *base = it->first;
         return true;
     }
-    uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes) override {
+    uintptr_t place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes, bool lines) override {
         uintptr_t base;
         if (!side_rule || !arena_of(lo, &base)) return 0;
         SideHash h;
         h.known = true;
         h.address_mask = side_mask;
-        return canonical_start(h, flip_of(base), base, lo, hi, bytes);
+        return canonical_start(h, flip_of(base), base, lo, hi, bytes, lines);
     }
     int side_of(uintptr_t addr) const {
         uintptr_t base;
