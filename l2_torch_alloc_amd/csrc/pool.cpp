@@ -135,6 +135,15 @@ bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* t
             placed = true;
             break;
         }
+        if (!placed) {
+            // the best fit after all, but at least on the right starting page: the block then follows
+            // the pattern up to the first 256 MiB line it meets
+            const uintptr_t at = backing_->place_canonical(sit->second, sit->second + sit->first, bytes, /*lines=*/false);
+            if (at != 0) {
+                assert(at >= sit->second && at + bytes <= sit->second + sit->first && at % kRegionAlign == 0);
+                start = at;
+            }
+        }
         if (placed) st_.canonical_placements++;
     }
     const uintptr_t ext_addr = sit->second;

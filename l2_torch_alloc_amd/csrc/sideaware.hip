@@ -728,9 +728,10 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
 
 // A sided launch follows its output.  An input that is as wide as the output and read at the
 // output's index is then on the right half of the device wherever its side pattern matches the
-// output's, and on the wrong half (every load crossing between the dies: a 256 MiB copy drops from
-// 6.9 to 6.3 TB/s, below the striped map's 6.7) wherever it does not.  True when every such input
-// lies in an arena of known sides and matches the output over at least nine tenths of the array
+// output's, and on the wrong half wherever it does not (every load crossing between the dies).
+// Measured with a 256 MiB copy: all matching 6.9 TB/s, none matching 6.3, the striped map 6.7, so the
+// sided map still wins with up to two fifths of the array mismatched.  True when every such input
+// lies in an arena of known sides and matches the output over at least seven tenths of the array
 // (the patterns are piecewise constant between carries into the hash bits: 64 samples see them).
 static bool inputs_follow_output(DeviceContext* ctx, const CompiledKernel* k, const void* out0, const void* const in[4],
                                  size_t num_bytes) {
@@ -754,7 +755,7 @@ static bool inputs_follow_output(DeviceContext* ctx, const CompiledKernel* k, co
             const unsigned int b = side_parity(((uintptr_t)out0 - out_base + off) & hash.address_mask) ^ out_flip;
             agree += a == b;
         }
-        if (agree * 10 < kSamples * 9) return false;
+        if (agree * 10 < kSamples * 7) return false;
     }
     return true;
 }

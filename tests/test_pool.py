@@ -513,18 +513,21 @@ def test_large_regions_share_one_side_pattern(ph):
             continue                                       # below the size the rule applies to, or a reused region
         fresh += 1
         if after["canonical_placements"] == before["canonical_placements"]:
-            continue                                       # no free run could hold it that way: plain best fit
+            # no free run could hold it that way without a large hole in front: the best fit, on the
+            # right starting page (it then follows the pattern up to the first 256 MiB line it meets)
+            assert ph.ph_side_of(p.h, ptr) == 0 and ph.ph_side_of(p.h, ptr + 8192) == 1
+            continue
         placed += 1
-        # up to a sixteenth of a region may lie past a line where the pattern flips
+        # up to an eighth of a region may lie past a line where the pattern flips
         hits = total = 0
         for _ in range(200):
             o = rng.randrange(0, n) & ~0x1fff
             hits += ph.ph_side_of(p.h, ptr + o) == bin(o & SIDE_BITS).count("1") & 1
             total += 1
-        assert hits >= 0.9 * total, (hex(ptr), n // MiB, hits, total)
+        assert hits >= 0.85 * total, (hex(ptr), n // MiB, hits, total)
         assert ph.ph_side_of(p.h, ptr) == 0 and ph.ph_side_of(p.h, ptr + 8192) == 1
         checked += total
-    assert placed >= 0.9 * fresh and placed > 50 and checked > 2000, (placed, fresh, checked)
+    assert placed >= 0.8 * fresh and placed > 50 and checked > 2000, (placed, fresh, checked)
     # blocks stay disjoint and inside what the backing store handed out
     spans = sorted(live)
     for (a, n), (b, _) in zip(spans, spans[1:]):
