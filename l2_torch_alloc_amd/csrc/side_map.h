@@ -149,7 +149,8 @@ private:
     void discover_locked();
     int probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream,
                         unsigned int* work);
-    bool measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides);
+    bool measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides,
+                        bool busy_device);
 
     int device_;
     std::mutex mu_;

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(64) void sa_side_classify(const unsigned int* lat, 
     int side = -1;
     if (ok) {
         const float lo = mid[0] < mid[1] ? mid[0] : mid[1], hi = mid[0] < mid[1] ? mid[1] : mid[0];
-        if (hi - lo >= 60.0f && hi - lo >= 0.1f * lo) side = mid[0] < mid[1] ? 0 : 1;
+        if (hi - lo >= 0.2f * lo) side = mid[0] < mid[1] ? 0 : 1;      // near about 450 cycles, far about 680
     }
     sides[i] = side;
 }
@@ -246,7 +246,8 @@ SideRegistry::~SideRegistry() {
 
 // Times loads at base + offsets[i] from every XCD and says, for each i, which half of the XCDs is
 // nearer: 0 (XCDs 0 .. n/2-1), 1, or -1 when the two halves do not differ clearly.
-bool SideRegistry::measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides) {
+bool SideRegistry::measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides,
+                                  bool busy_device) {
     const int n = (int)offsets.size();
     sides->assign(n, -1);
     if (n == 0 || n > kMaxProbe || bytes < kScrubBytes) return false;
@@ -302,10 +303,10 @@ bool SideRegistry::measure_locked(const char* base, size_t bytes, const std::vec
         }
         const double a = mid[0], b = mid[1];
         const double lo = a < b ? a : b, hi = a < b ? b : a;
-        // idle: near about 450 cycles, far about 680; with other kernels running both rise (740 / 880):
-        // a tenth apart, and at least 60 cycles, still tells the halves apart, and the votes that
-        // use these answers tolerate a few wrong ones
-        const bool clear = hi - lo >= 60.0 && hi - lo >= 0.1 * lo;
+        // Idle: near about 450 cycles, far about 680: a fifth apart is clear.  With other kernels
+        // running both rise (740 / 880): a tenth apart, and at least 60 cycles, still tells the halves
+        // apart most of the time, which is good enough for a vote that tolerates a few wrong answers.
+        const bool clear = busy_device ? (hi - lo >= 60.0 && hi - lo >= 0.1 * lo) : (hi - lo >= 0.2 * lo);
         if (side_debug() && !clear) {
             std::fprintf(stderr, "sideaware: probe %3d at +0x%llx:", i, (unsigned long long)offsets[i]);
             for (int x = 0; x < kProbeGroups; x++) std::fprintf(stderr, " %u", lat[(size_t)x * n + i]);
@@ -350,7 +351,7 @@ void SideRegistry::discover_locked() {
         }
     }
     std::vector<int> sides;
-    const bool measured = measure_locked(scratch, kBytes, offsets, &sides);
+    const bool measured = measure_locked(scratch, kBytes, offsets, &sides, /*busy_device=*/false);
     (void)hipFree(scratch);
     if (!measured) {
         if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: the probe could not run\n");
@@ -397,7 +398,7 @@ void SideRegistry::vote_locked(ArenaSide& a) {
         offsets.push_back(gi << kSideGranuleLog2);
     }
     std::vector<int> sides;
-    if (!measure_locked((const char*)a.base, a.bytes, offsets, &sides)) return;
+    if (!measure_locked((const char*)a.base, a.bytes, offsets, &sides, /*busy_device=*/true)) return;
     int votes[2] = {0, 0};
     for (int i = 0; i < kSamples; i++) {
         if (sides[i] < 0) continue;

@@ -102,6 +102,30 @@ def test_which_launches_are_sided(sa, lib):
     # in place: the input is the output
     assert copy(dst.data_ptr(), dst.data_ptr(), n) == (1, 0)
     assert torch.equal(dst, src)
+    # an op whose only input is narrower than its output is faster on the striped map; one with no
+    # input at all follows its output
+    widen = sa.sideaware_create_kernel(b"""
+typedef float o0;
+typedef __bf16 i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband, o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) { out0 = (float)in0; }
+""")
+    x = torch.randn(16 * MiB, device="cuda").to(torch.bfloat16)
+    y = torch.empty(16 * MiB, device="cuda")
+    before = counts(lib)
+    lib.sideaware_one_to_one(widen, y.numel() * 4, y.data_ptr(), x.data_ptr(), 0, stream)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0], before[1] + 1) and torch.equal(y, x.float())
+    from l2_torch_alloc_amd import ops
+    z = torch.empty(16 * MiB, dtype=torch.int32, device="cuda")
+    before = counts(lib)
+    ops.fill_int32(z, 7)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0] + 1, before[1]) and bool((z == 7).all())
 
 
 def agreeing_offset(lib, base, nbytes, first):
