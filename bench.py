@@ -512,9 +512,13 @@ def bench_churn(use_sideaware, n_ops=10000, live_cap=64 * GiB):
         else:
             torch.add(x * 1.5, 0.25, out=y)
 
-    # Untimed: one op per size and alignment class, so that no first-use compile (the library
-    # builds an instantiation per class on first use) or lazy initialisation of PyTorch's kernels
-    # falls between the events of a sampled op below.
+    # Untimed: every instantiation of the op is built ahead (the library builds one per size,
+    # alignment and ownership class on first use), and one op per size and alignment class is run,
+    # so that no first-use compile or lazy initialisation of PyTorch's kernels falls between the
+    # events of a sampled op below.
+    if use_sideaware:
+        from l2_torch_alloc_amd import headers, wrapper
+        wrapper.library().sideaware_create_kernel_advanced(headers.scale_bias_bf16_header(), True, 0)
     for size in (4096, 3 * MiB + 4096, 64 * MiB, 300 * MiB):
         pad = torch.empty(size // 2 + 256, dtype=torch.bfloat16, device="cuda")
         for x in (torch.empty(size // 2, dtype=torch.bfloat16, device="cuda"), pad[256:]):

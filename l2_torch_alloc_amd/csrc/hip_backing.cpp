@@ -77,7 +77,7 @@ void HipBacking::release(void* ptr, size_t) {
 uintptr_t HipBacking::place_canonical(uintptr_t lo, uintptr_t hi, size_t bytes, bool lines) {
     uintptr_t base = 0;
     unsigned int flip = 0;
-    if (!sides_.arena_of((const void*)lo, &base, &flip)) return 0;
+    if (!sides_.arena_of((const void*)lo, &base, &flip, /*placing=*/true)) return 0;
     return canonical_start(sides_.hash(), flip, base, lo, hi, bytes, lines);
 }
 

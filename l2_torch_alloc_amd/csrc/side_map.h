@@ -112,8 +112,9 @@ public:
     bool lookup(const void* addr, size_t bytes, SideMap* out);
     // Side of the granule at addr: 0, 1, or -1 when unknown.
     int side_of(const void* addr);
-    // Arena constants for the placement rule: false when addr is in no known arena.
-    bool arena_of(const void* addr, uintptr_t* base, unsigned int* flip);
+    // Arena constants: false when addr is in no known arena.  `placing` says the caller is the pool
+    // placing a region: an arena whose first measurement was inconclusive is then measured again.
+    bool arena_of(const void* addr, uintptr_t* base, unsigned int* flip, bool placing = false);
 
     // Where workgroup 0 of a sided launch on `stream` reports its XCD (pinned host memory the
     // device can write), and the dealing offset last reported there (0 before the first report).

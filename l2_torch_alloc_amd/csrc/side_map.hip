@@ -427,11 +427,12 @@ void SideRegistry::add_arena(void* base, size_t bytes) {
     arenas_.push_back(a);
 }
 
-// An arena whose vote was inconclusive is measured again when somebody asks about it, a few times at
-// most and not on every question.
+// An arena whose vote was inconclusive is measured again when the pool next places a region in
+// it (an allocation that carves is a slow path already; launches never wait for a probe), a few
+// times at most and not on every placement.
 void SideRegistry::maybe_vote_again_locked(ArenaSide& a) {
     if (a.known || a.tries >= kMaxVoteTries) return;
-    if (++a.asked % 16 != 0) return;
+    if (++a.asked % 4 != 0) return;
     vote_locked(a);
 }
 
@@ -462,9 +463,8 @@ bool SideRegistry::lookup(const void* addr, size_t bytes, SideMap* out) {
     const uintptr_t p = (uintptr_t)addr;
     std::lock_guard<std::mutex> g(mu_);
     if (!hash_.known) return false;
-    for (ArenaSide& a : arenas_) {
+    for (const ArenaSide& a : arenas_) {
         if (p >= a.base && p - a.base < a.bytes) {
-            maybe_vote_again_locked(a);
             if (!a.known || bytes > a.bytes - (p - a.base)) return false;
             out->origin_address = a.base;
             out->pair_mask = hash_.pair_mask();
@@ -475,12 +475,13 @@ bool SideRegistry::lookup(const void* addr, size_t bytes, SideMap* out) {
     return false;
 }
 
-bool SideRegistry::arena_of(const void* addr, uintptr_t* base, unsigned int* flip) {
+bool SideRegistry::arena_of(const void* addr, uintptr_t* base, unsigned int* flip, bool placing) {
     const uintptr_t p = (uintptr_t)addr;
     std::lock_guard<std::mutex> g(mu_);
     if (!hash_.known) return false;
-    for (const ArenaSide& a : arenas_) {
+    for (ArenaSide& a : arenas_) {
         if (p >= a.base && p - a.base < a.bytes) {
+            if (placing) maybe_vote_again_locked(a);
             if (!a.known) return false;
             *base = a.base;
             *flip = a.flip;

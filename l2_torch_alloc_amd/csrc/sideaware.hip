@@ -874,6 +874,12 @@ int sideaware_create_kernel_advanced(const char* header, bool precompile, int de
                                        kVariantUnaligned, kVariantUnaligned | kVariantInPlace,
                                        kVariantUnaligned | kVariantBeyond};
             for (int v : kAll) get_kernel(ctx, id, v);
+            // ... and the same with the sided ownership map, for ops that can follow their output
+            KernelEntry* e = find_entry(id);
+            for (int v : kAll) {
+                if (e && e->sided_possible.load(std::memory_order_relaxed) == 0) break;
+                get_kernel(ctx, id, v | kVariantSided);
+            }
         }
     }
     return id;
