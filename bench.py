@@ -148,7 +148,7 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
             "frac_of_peak": gbps(2 * nbytes, sec) / HBM_PEAK_GBPS, "bit_exact": ok}
 
 
-def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4):
+def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4, named_kernels=False):
     """The 256 MiB cycling copy under the three ownership maps, timed in turn `rounds` times over
     (medians): sided (every XCD moves the granules of its own half of the device), XCD-striped
     (the map that needs no knowledge of the halves), and sided the wrong way round (every access
@@ -162,10 +162,22 @@ def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4):
     ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
     counter = [0]
 
+    # for a kernel trace: the same copy under three names, one per setting
+    kids = {}
+    if named_kernels:
+        from l2_torch_alloc_amd import headers, wrapper
+        for name in ("sided", "xcd_striped", "sided_wrong_way_round"):
+            text = headers.memcpy_header().decode().replace("sideaware_copy_spelled_out", "sideaware_copy_" + name)
+            kids[name] = wrapper.sideaware_create_kernel(text.encode())
+    current = [None]
+
     def launch():
         d_ptr, s_ptr = ptrs[counter[0] % pairs]
         counter[0] += 1
-        lib.sideaware_memcpy(d_ptr, s_ptr, nbytes, 0, stream)
+        if named_kernels:
+            lib.sideaware_one_to_one(kids[current[0]], nbytes, d_ptr, s_ptr, 0, stream)
+        else:
+            lib.sideaware_memcpy(d_ptr, s_ptr, nbytes, 0, stream)
 
     def launches():
         a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
@@ -180,6 +192,7 @@ def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4):
             for name, sided, wrong in settings:
                 lib.sideaware_tune(b"sided", sided)
                 lib.sideaware_tune(b"sided_wrong", wrong)
+                current[0] = name
                 before = launches()
                 times[name].append(time_region(launch, steps, pairs))
                 after = launches()
@@ -745,6 +758,9 @@ def main():
                          "(for per-XCD TCC hit rates)")
     ap.add_argument("--launch-shapes", action="store_true",
                     help="only the library's copy and bf16 RoPE over every ownership stripe, buffers cycling")
+    ap.add_argument("--side-ab", action="store_true",
+                    help="only the 256 MiB copy under the three ownership maps (sided, XCD-striped, sided the wrong "
+                         "way round), each under a kernel name of its own (for a kernel trace)")
     ap.add_argument("--only", action="append", default=None,
                     help="with an experiment mode: run only the cases whose name contains this text")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
@@ -773,6 +789,9 @@ def main():
     if any((args.stripe_ab, args.inflight_ab, args.cache_probe, args.chain_policy, args.chain_xcd, args.launch_shapes,
             args.ceiling)):
         import bench_experiments as experiments      # the sweep modes: not needed by the default run
+    if args.side_ab:
+        print(json.dumps({"copy_256MiB_ownership_map_ab": bench_side_ab(named_kernels=True)}))
+        return
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": experiments.stripe_ab(args.steps)}))
         return
