@@ -129,6 +129,8 @@ public:
     int probe_sides(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream,
                     bool allocate);
     void init_static_scratch();
+    // Allocates the feedback words ahead of the first sided launch (feedback_slot does it otherwise).
+    void init_feedback();
     static constexpr int kNoAllocMaxSamples = 512;
 
     // For tests and tools: forget what was measured / pretend.
@@ -148,6 +150,7 @@ private:
     void vote_locked(ArenaSide& a);
     void maybe_vote_again_locked(ArenaSide& a);
     void discover_locked();
+    bool ensure_feedback_locked();
     int probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides, void* stream,
                         unsigned int* work);
     bool measure_locked(const char* base, size_t bytes, const std::vector<uint64_t>& offsets, std::vector<int>* sides,

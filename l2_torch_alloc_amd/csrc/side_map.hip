@@ -180,6 +180,26 @@ void SideRegistry::init_static_scratch() {
     static_scratch_ = (unsigned int*)ptr;            // this device's copy of the array
 }
 
+// The pinned words the sided kernels report their XCD to.  Allocated when the device is set up, so
+// that a first sided launch may happen under stream capture (which allows no allocation).
+bool SideRegistry::ensure_feedback_locked() {
+    if (feedback_) return true;
+    DeviceGuard dev(device_);
+    void* p = nullptr;
+    if (hipHostMalloc(&p, kFeedbackSlots * 64, hipHostMallocMapped) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    std::fill_n((unsigned int*)p, kFeedbackSlots * 16, 0u);
+    feedback_ = (volatile unsigned int*)p;
+    return true;
+}
+
+void SideRegistry::init_feedback() {
+    std::lock_guard<std::mutex> g(mu_);
+    (void)ensure_feedback_locked();
+}
+
 // The probe behind sideaware_probe_sides and sideaware_probe_sides_noalloc: everything runs on the
 // caller's stream, the results stay on the device.  `work` holds 16 * count + 16 words.
 int SideRegistry::probe_on_stream(const void* region, size_t bytes, unsigned long long seed, int count, int* sides,
@@ -319,8 +339,11 @@ bool SideRegistry::measure_locked(const char* base, size_t bytes, const std::vec
 }
 
 // Which address bits decide the side?  For every candidate bit, a few granules and their partners
-// with that bit flipped: a bit is in the hash when every pair lands on different sides, out of it
-// when none does, and the whole discovery fails on anything in between.
+// with that bit flipped: a bit is in the hash when (all but at most one of) the pairs land on
+// different sides, out of it when (all but at most one) land on the same side, and an attempt fails on
+// anything in between.  A failed attempt (timings disturbed by whatever else the device was doing)
+// is repeated with other sample granules, a few times; a device that has no such structure fails
+// every time and is then treated as one-sided for the life of the process.
 void SideRegistry::discover_locked() {
     if (discovered_) return;
     discovered_ = true;
@@ -334,45 +357,50 @@ void SideRegistry::discover_locked() {
         return;
     }
     constexpr size_t kBytes = 1ull << 30;
-    constexpr int kLowBit = 12, kHighBit = 29, kPairsPerBit = 8, kPairsNeeded = 5;
+    constexpr int kLowBit = 12, kHighBit = 29, kPairsPerBit = 8, kPairsNeeded = 5, kAttempts = 3;
     size_t free_bytes = 0, total = 0;
     if (hipMemGetInfo(&free_bytes, &total) != hipSuccess || free_bytes < 2 * kBytes) { (void)hipGetLastError(); return; }
     char* scratch = nullptr;
     if (hipMalloc((void**)&scratch, kBytes) != hipSuccess) { (void)hipGetLastError(); return; }
-    std::vector<uint64_t> offsets;
     uint64_t lcg = 0x9e3779b97f4a7c15ull;
-    for (int b = kLowBit; b <= kHighBit; b++) {
-        for (int j = 0; j < kPairsPerBit; j++) {
-            lcg = lcg * 6364136223846793005ull + 1442695040888963407ull;
-            uint64_t x = (lcg >> 20) % kBytes;
-            x &= ~((1ull << kLowBit) - 1) & ~(1ull << b);
-            offsets.push_back(x);
-            offsets.push_back(x | (1ull << b));
+    for (int attempt = 1; attempt <= kAttempts && !hash_.known; attempt++) {
+        std::vector<uint64_t> offsets;
+        for (int b = kLowBit; b <= kHighBit; b++) {
+            for (int j = 0; j < kPairsPerBit; j++) {
+                lcg = lcg * 6364136223846793005ull + 1442695040888963407ull;
+                uint64_t x = (lcg >> 20) % kBytes;
+                x &= ~((1ull << kLowBit) - 1) & ~(1ull << b);
+                offsets.push_back(x);
+                offsets.push_back(x | (1ull << b));
+            }
         }
+        std::vector<int> sides;
+        if (!measure_locked(scratch, kBytes, offsets, &sides, /*busy_device=*/false)) {
+            if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: the probe could not run\n");
+            break;
+        }
+        uint64_t mask = 0;
+        size_t at = 0;
+        bool consistent = true;
+        for (int b = kLowBit; b <= kHighBit; b++) {
+            int flips = 0, same = 0;
+            for (int j = 0; j < kPairsPerBit; j++, at += 2) {
+                if (sides[at] < 0 || sides[at + 1] < 0) continue;
+                (sides[at] != sides[at + 1] ? flips : same)++;
+            }
+            if (side_debug()) {
+                std::fprintf(stderr, "sideaware: side discovery, attempt %d: bit %d: %d pairs flip, %d do not\n", attempt, b,
+                             flips, same);
+            }
+            if (flips >= kPairsNeeded && same <= 1) mask |= 1ull << b;
+            else if (!(same >= kPairsNeeded && flips <= 1)) consistent = false;      // not a parity of address bits
+        }
+        // the kernels assume granules of exactly 8 KiB
+        if (!consistent || !((mask >> kSideGranuleLog2) & 1) || (mask & ((1ull << kSideGranuleLog2) - 1))) continue;
+        hash_.known = true;
+        hash_.address_mask = mask;
     }
-    std::vector<int> sides;
-    const bool measured = measure_locked(scratch, kBytes, offsets, &sides, /*busy_device=*/false);
     (void)hipFree(scratch);
-    if (!measured) {
-        if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: the probe could not run\n");
-        return;
-    }
-    uint64_t mask = 0;
-    size_t at = 0;
-    for (int b = kLowBit; b <= kHighBit; b++) {
-        int flips = 0, same = 0;
-        for (int j = 0; j < kPairsPerBit; j++, at += 2) {
-            if (sides[at] < 0 || sides[at + 1] < 0) continue;
-            (sides[at] != sides[at + 1] ? flips : same)++;
-        }
-        if (side_debug()) std::fprintf(stderr, "sideaware: side discovery: bit %d: %d pairs flip, %d do not\n", b, flips, same);
-        if (flips >= kPairsNeeded && same == 0) mask |= 1ull << b;
-        else if (!(same >= kPairsNeeded && flips == 0)) return;              // not a parity of address bits
-    }
-    // the kernels assume granules of exactly 8 KiB
-    if (!((mask >> kSideGranuleLog2) & 1) || (mask & ((1ull << kSideGranuleLog2) - 1))) return;
-    hash_.known = true;
-    hash_.address_mask = mask;
 }
 
 void SideRegistry::discover() {
@@ -502,16 +530,7 @@ int SideRegistry::side_of(const void* addr) {
 unsigned int* SideRegistry::feedback_slot(void* stream, unsigned int* dealing) {
     std::lock_guard<std::mutex> g(mu_);
     *dealing = 0;
-    if (!feedback_) {
-        DeviceGuard dev(device_);
-        void* p = nullptr;
-        if (hipHostMalloc(&p, kFeedbackSlots * 64, hipHostMallocMapped) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
-        }
-        std::fill_n((unsigned int*)p, kFeedbackSlots * 16, 0u);
-        feedback_ = (volatile unsigned int*)p;
-    }
+    if (!ensure_feedback_locked()) return nullptr;
     int slot;
     auto it = slot_of_stream_.find(stream);
     if (it != slot_of_stream_.end()) {

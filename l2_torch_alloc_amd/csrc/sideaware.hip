@@ -333,6 +333,7 @@ void DeviceContext::initialize() {
     backing = std::make_unique<HipBacking>(device);
     backing->sides().discover();                 // which address bits decide the half of the device (a few ms)
     backing->sides().init_static_scratch();      // this device's address of the allocation-free probe's work array
+    backing->sides().init_feedback();            // before any launch, which may be under stream capture
     side_summary[4] = side_hash_mask(this);
     pool = std::make_unique<Pool>(backing.get());
     // The reference trims its cache from 16 GiB down to 2 GiB on an 80 GB part

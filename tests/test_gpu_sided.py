@@ -203,6 +203,39 @@ def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
     assert 0 <= lib.sideaware_stream_dealing(stream) <= 7
 
 
+def test_sided_launches_replay_from_a_hip_graph(sa, lib):
+    """A sided launch under stream capture: the dealing offset the host believed at capture time
+    is frozen into the graph's kernel arguments; whatever the stream does on later replays, every
+    replay is bit-exact (the map is a bijection for any belief), also with eager work between them."""
+    n = 64 * MiB
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    mid = torch.zeros_like(src)
+    dst = torch.zeros_like(src)
+    torch.ops.sideaware.memcpy(mid, src)            # compiles the instantiation outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    before = counts(lib)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            torch.ops.sideaware.memcpy(mid, src)
+            torch.ops.sideaware.memcpy(dst, mid)
+    torch.cuda.current_stream().wait_stream(side)
+    assert counts(lib)[0] == before[0] + 2, "the captured launches were not sided"
+    other = torch.zeros(16 * MiB, dtype=torch.uint8, device="cuda")
+    for trial in range(4):
+        src.random_(0, 256)
+        dst.zero_()
+        torch.ops.sideaware.memcpy(other, src[: 16 * MiB])      # eager work of the program's own between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dst, src), trial
+        assert torch.equal(other, src[: 16 * MiB]), trial
+    assert not sa.sideaware_last_error()
+
+
 def test_sided_elementwise_with_two_inputs_and_mixed_widths(sa, lib):
     """bf16 x -> fp32 y (the output is the wider array, so the map follows it) and a two-input
     fp32 op, both compared with torch."""
