@@ -212,7 +212,8 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * "one_shot", "cache_bytes" (launch parameters) and "nt_store", "wg_threads", "write_through"
  * (1: stores are written through the XCD's private L2; 0: the compiler's write-back stores)
  * (compiled in: after a change every op is compiled afresh on its next launch); "sided" (1: launches
- * whose output lies in an arena of known sides use the sided map, 0: never), "sided_min_bytes" (arrays
+ * whose first output (first input, for an op whose output is narrower) lies in an arena of known sides use
+ * the sided map, 0: never), "sided_min_bytes" (arrays
  * shorter than this never do), "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
  * -1: by array size) and "sided_wrong" (1: sided launches give every XCD the granules of the other half
  * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,

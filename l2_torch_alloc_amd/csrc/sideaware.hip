@@ -711,62 +711,82 @@ static long long slots_wanted_for(const DeviceContext* ctx, const CompiledKernel
     return (long long)per_xcd * groups;
 }
 
-// Whether a launch whose first output is [out0, out0 + num_bytes) may use the sided map, and with
-// which arena constants: the output must lie in an arena whose sides were measured, start on a
-// granule boundary and be long enough to matter, and the op must be one that can follow its
-// output (see sa_sided_possible in the kernel template).
-static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const void* out0, size_t num_bytes,
-                            const Tuning& t, SideMap* map) {
-    if (!t.sided || out0 == nullptr || num_bytes < (unsigned long long)t.sided_min_bytes) return false;
-    if (((uintptr_t)out0 & ((1u << kSideGranuleLog2) - 1)) != 0) return false;
+// Whether it is worth looking at the sided instantiation of an op for this launch at all: the map
+// is switched on, the array is long enough to matter, the op is not known to be one that cannot be
+// sided (see sa_sided_possible in the kernel template), and one of the two arrays a sided launch may
+// follow starts on a granule boundary in an arena whose sides were measured.
+static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const void* out0, const void* in0,
+                            size_t num_bytes, const Tuning& t) {
+    if (!t.sided || num_bytes < (unsigned long long)t.sided_min_bytes) return false;
     if (entry->sided_possible.load(std::memory_order_relaxed) == 0) return false;
     if (ctx->num_xcds < 2 || (ctx->num_xcds & (ctx->num_xcds - 1))) return false;
-    if (!ctx->backing->sides().lookup(out0, num_bytes, map)) return false;
-    // The counterpart of the reference's FORCE_WRONG_SIDE (sideaware.cu:70-75, 297-298): the same
-    // map with the arena's constant inverted, so that every access crosses to the other half.
-    if (t.sided_wrong) map->flip ^= 1u;
-    return true;
+    constexpr uintptr_t kGranuleMask = (1u << kSideGranuleLog2) - 1;
+    SideRegistry& sides = ctx->backing->sides();
+    uintptr_t base = 0;
+    unsigned int flip = 0;
+    for (const void* p : {out0, in0}) {
+        if (p && ((uintptr_t)p & kGranuleMask) == 0 && sides.arena_of(p, &base, &flip)) return true;
+    }
+    return false;
 }
 
-// A sided launch follows its output.  An input that is as wide as the output and read at the
-// output's index is then on the right half of the device wherever its side pattern matches the
-// output's, and on the wrong half wherever it does not (every load crossing between the dies).
-// Measured with a 256 MiB copy: all matching 6.9 TB/s, none matching 6.3, the striped map 6.7, so the
-// sided map still wins with up to two fifths of the array mismatched.  True when every such input
-// lies in an arena of known sides and matches the output over at least seven tenths of the array
-// (the patterns are piecewise constant between carries into the hash bits: 64 samples see them).
-static bool inputs_follow_output(DeviceContext* ctx, const CompiledKernel* k, const void* out0, const void* const in[4],
-                                 size_t num_bytes) {
+// Whether this launch of the sided instantiation `k` may go ahead, and with which arena constants.
+// A sided launch follows one array, the wider of o0 and i0 (o0 when they are as wide as each other;
+// num_bytes is that array's length): it must lie in an arena whose sides were measured and start on
+// a granule boundary.  Every other array that is as wide and accessed at the same index (outputs;
+// inputs unless gathered through a custom `indexing`) is then on the right half of the device
+// wherever its side pattern matches the followed array's, and on the wrong half wherever it does not
+// (every access crossing between the dies).  Measured with a 256 MiB copy: all matching 6.9 TB/s, none
+// matching 6.3, the striped map 6.7, so the sided map still wins with up to two fifths of the array
+// mismatched.  Such an array must therefore lie in an arena of known sides and match over at least
+// seven tenths of its length (the patterns are piecewise constant between carries into the hash
+// bits: 64 samples see them).  Narrower arrays fall where they fall: half of their traffic crosses.
+static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const void* const out[4], const void* const in[4],
+                            size_t num_bytes, const Tuning& t, SideMap* map) {
     SideRegistry& sides = ctx->backing->sides();
+    const void* owner = k->owner_is_o0 ? out[0] : in[0];
+    const int owner_size = k->owner_is_o0 ? k->out_size[0] : k->in_size[0];
+    if (owner == nullptr || owner_size == 0 || ((uintptr_t)owner & ((1u << kSideGranuleLog2) - 1)) != 0) return false;
+    if (!sides.lookup(owner, num_bytes, map)) return false;
     const SideHash hash = sides.hash();
-    uintptr_t out_base = 0;
-    unsigned int out_flip = 0;
-    if (!sides.arena_of(out0, &out_base, &out_flip)) return false;
+    uintptr_t owner_base = 0;
+    unsigned int owner_flip = 0;
+    if (!sides.arena_of(owner, &owner_base, &owner_flip)) return false;
+    auto follows = [&](const void* p) {
+        if (p == owner) return true;                                   // in place
+        uintptr_t base = 0;
+        unsigned int flip = 0;
+        if (!sides.arena_of(p, &base, &flip)) return false;
+        constexpr int kSamples = 64;
+        int agree = 0;
+        for (int i = 0; i < kSamples; i++) {
+            const uint64_t off = (uint64_t)(num_bytes / kSamples) * (unsigned)i;
+            const unsigned int a = side_parity(((uintptr_t)p - base + off) & hash.address_mask) ^ flip;
+            const unsigned int b = side_parity(((uintptr_t)owner - owner_base + off) & hash.address_mask) ^ owner_flip;
+            agree += a == b;
+        }
+        return agree * 10 >= kSamples * 7;
+    };
     bool any_input = false, any_as_wide = false;
     for (int j = 0; j < 4; j++) {
         if (!in[j] || k->in_size[j] == 0) continue;
         if (j > 0 && k->gathered) continue;
         any_input = true;
-        if (k->in_size[j] != k->out_size[0]) continue;
+        if (k->in_size[j] != owner_size) continue;
         any_as_wide = true;
-        if (in[j] == out0) continue;                                   // in place
-        uintptr_t in_base = 0;
-        unsigned int in_flip = 0;
-        if (!sides.arena_of(in[j], &in_base, &in_flip)) return false;
-        constexpr int kSamples = 64;
-        int agree = 0;
-        for (int i = 0; i < kSamples; i++) {
-            const uint64_t off = (uint64_t)(num_bytes / kSamples) * (unsigned)i;
-            const unsigned int a = side_parity(((uintptr_t)in[j] - in_base + off) & hash.address_mask) ^ in_flip;
-            const unsigned int b = side_parity(((uintptr_t)out0 - out_base + off) & hash.address_mask) ^ out_flip;
-            agree += a == b;
-        }
-        if (agree * 10 < kSamples * 7) return false;
+        if (!follows(in[j])) return false;
+    }
+    for (int j = 0; j < 4; j++) {
+        if (!out[j] || k->out_size[j] != owner_size) continue;
+        if (!follows(out[j])) return false;
     }
     // An op that only widens (every input narrower than the output: an MXFP8 -> bf16 dequantise)
     // loses with the sided map, 6.1 against 6.4 TB/s: the halves of each of its input granules go to
     // XCDs of different sides.  An op with no input at all (a fill) only gains.
     if (any_input && !any_as_wide) return false;
+    // The counterpart of the reference's FORCE_WRONG_SIDE (sideaware.cu:70-75, 297-298): the same
+    // map with the arena's constant inverted, so that every access crosses to the other half.
+    if (t.sided_wrong) map->flip ^= 1u;
     return true;
 }
 
@@ -909,11 +929,13 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     if (!entry) return;
     SideMap side;
     const CompiledKernel* k = nullptr;
-    if (sided_candidate(ctx, entry, out0, num_bytes, t, &side)) {
+    if (sided_candidate(ctx, entry, out0, in0, num_bytes, t)) {
         k = get_kernel(ctx, kernel_id, variant | kVariantSided);
+        const void* const outs[4] = {out0, out1, out2, out3};
         const void* const ins[4] = {in0, in1, in2, in3};
-        // the op cannot follow its output, or an input lies across from it: the striped map
-        if (k && (!k->sided || !inputs_follow_output(ctx, k, out0, ins, num_bytes))) k = nullptr;
+        // the op cannot be sided, the array it follows is not in measured memory, or another array
+        // lies across from that one: the striped map
+        if (k && (!k->sided || !sided_launch_ok(ctx, k, outs, ins, num_bytes, t, &side))) k = nullptr;
     }
     if (!k) k = get_kernel(ctx, kernel_id, variant);
     if (!k) return;
@@ -924,8 +946,8 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     LaunchPlan plan;
     if (k->sided) {
         feedback = ctx->backing->sides().feedback_slot(stream, &side.dealing);
-        plan = plan_launch_sided((uint64_t)(uintptr_t)out0, num_vectors, k->tile_vectors, ctx->num_xcds,
-                                 sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side);
+        plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0), num_vectors, k->tile_vectors,
+                                 ctx->num_xcds, sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side);
     } else {
         const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0);
         plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,
@@ -1016,14 +1038,14 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
         SideMap sides[kMaxSegments];
         bool all_sided = true;
         for (int i = 0; i < count && all_sided; i++) {
-            all_sided = sided_candidate(ctx, entry, group[i]->out[0], group[i]->num_bytes, t, &sides[i]);
+            all_sided = sided_candidate(ctx, entry, group[i]->out[0], group[i]->in[0], group[i]->num_bytes, t);
         }
         const CompiledKernel* k = nullptr;
         if (all_sided) {
             k = get_kernel(ctx, kernel_id, variant | kVariantSided);
             if (k && !k->sided) k = nullptr;
             for (int i = 0; i < count && k; i++) {
-                if (!inputs_follow_output(ctx, k, group[i]->out[0], group[i]->in, group[i]->num_bytes)) k = nullptr;
+                if (!sided_launch_ok(ctx, k, group[i]->out, group[i]->in, group[i]->num_bytes, t, &sides[i])) k = nullptr;
             }
         }
         if (!k) k = get_kernel(ctx, kernel_id, variant);
@@ -1042,7 +1064,8 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
             LaunchPlan plan;
             if (k->sided) {
                 sides[i].dealing = dealing;
-                plan = plan_launch_sided((uint64_t)(uintptr_t)g.out[0], num_vectors, k->tile_vectors, ctx->num_xcds,
+                plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]), num_vectors,
+                                         k->tile_vectors, ctx->num_xcds,
                                          sided_stripe_for(g.num_bytes, g.out[0] == g.in[0], t), t.slot_run, slots_wanted, sides[i]);
             } else {
                 const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]);

@@ -352,7 +352,7 @@ def scale_bias_bf16_header(unrolled: int | None = None, evict_input: bool = True
     return "".join(lines).encode()
 
 
-def mxfp8_quantize_header(unrolled: int | None = 2) -> bytes:
+def mxfp8_quantize_header(unrolled: int | None = 1) -> bytes:
     """bf16 -> MXFP8 (OCP Microscaling: E4M3 elements with one E8M0 scale byte per 32 elements).
 
     The op the reference cites as the reason for its ``vector_op`` hook and sideband pointer

@@ -12,6 +12,8 @@
 //   visited exactly once" is the same as "each element ends at seed + 1".
 // SA_CASE_MIXED: four arrays of different element widths; checks that narrow and wide arrays are
 //   addressed with the same element index and that element_idx counts elements of the array.
+// SA_CASE_NARROW: float in, short out: the input is the wider array, so ownership (striped or sided)
+//   follows i0's address.
 #include <cstdio>
 #include <cstdlib>
 
@@ -148,6 +150,20 @@ static int run_case(unsigned grid, long long nv, size_t off) {
     }
     return bad;
 }
+#elif defined(SA_CASE_NARROW)
+static int run_case(unsigned grid, long long nv, size_t off) {
+    const size_t n = (size_t)nv * vec_size;
+    // i0 is the wider array: it is the one shifted by `off` and the one the ownership map follows
+    Arena f_in(off, n * sizeof(float)), s_out(off / 2, n * sizeof(short));
+    float* fi = (float*)f_in.data;
+    for (size_t i = 0; i < n; i++) fi[i] = (float)(i % 3001);
+    std::memset(s_out.data, 0xff, n * sizeof(short));
+    run_grid(grid, (size_type)nv, (vo0*)s_out.data, nullptr, nullptr, nullptr, (const vi0*)fi, nullptr, nullptr, nullptr,
+             nullptr, 0);
+    int bad = !s_out.sentinel_ok() + !f_in.sentinel_ok();
+    for (size_t i = 0; i < n; i++) bad += (((short*)s_out.data)[i] != (short)(i % 3001) + 1);
+    return bad;
+}
 #elif defined(SA_CASE_ROPE)
 // The op header under test is a generated RoPE header; rope_T / rope_half / rope_heads /
 // rope_rotated come from it.  The activation holds `nv` vectors (any length: a whole number of
@@ -194,7 +210,7 @@ static int run_case(unsigned grid, long long nv, size_t off) {
     return bad;
 }
 #else
-#error "define SA_CASE_INCREMENT, SA_CASE_MIXED or SA_CASE_ROPE"
+#error "define SA_CASE_INCREMENT, SA_CASE_MIXED, SA_CASE_NARROW or SA_CASE_ROPE"
 #endif
 
 int main() {

@@ -33,6 +33,24 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
 }
 """
 
+# A narrowing op (float in, short out): every output element is the id of the XCD its workgroup ran on.
+NARROWING_XCD_ID_HEADER = b"""
+#define KERNEL_NAME sideaware_test_narrowing_xcd_id
+typedef short o0;
+typedef float i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
+                                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    out0 = (short)((xcc & 0xf) + (in0 != 0.0f ? 100 : 0));
+}
+"""
+
 
 def counts(lib):
     a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
@@ -126,6 +144,19 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
     ops.fill_int32(z, 7)
     torch.cuda.synchronize()
     assert counts(lib) == (before[0] + 1, before[1]) and bool((z == 7).all())
+    # an op whose output is narrower than its input follows the input: the input must be in measured
+    # memory and start on a granule boundary, the output may be anywhere
+    narrow = sa.sideaware_create_kernel(NARROWING_XCD_ID_HEADER)
+    w = torch.zeros(16 * MiB, device="cuda")
+    h = torch.empty(16 * MiB + 8, dtype=torch.int16, device="cuda")
+    before = counts(lib)
+    lib.sideaware_one_to_one(narrow, w.numel() * 4, h.data_ptr() + 16, w.data_ptr(), 0, stream)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0] + 1, before[1])
+    before = counts(lib)
+    lib.sideaware_one_to_one(narrow, w.numel() * 4 - 8192, h.data_ptr(), w.data_ptr() + 4096, 0, stream)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0], before[1] + 1)
 
 
 def agreeing_offset(lib, base, nbytes, first):
@@ -233,6 +264,34 @@ def test_sided_launches_replay_from_a_hip_graph(sa, lib):
         torch.cuda.synchronize()
         assert torch.equal(dst, src), trial
         assert torch.equal(other, src[: 16 * MiB]), trial
+    assert not sa.sideaware_last_error()
+
+
+def test_a_narrowing_op_runs_on_the_side_of_its_input(sa, lib):
+    """float in, short out: the sided map follows the input (the wider array, two thirds of the
+    traffic).  Every 8 KiB granule of the input is read, and its 4 KiB of output written, by an XCD
+    of the half of the device that holds that input granule."""
+    stream = torch.cuda.current_stream().cuda_stream
+    kid = sa.sideaware_create_kernel(NARROWING_XCD_ID_HEADER)
+    n = 16 * MiB                                   # elements: 64 MiB in, 32 MiB out
+    src = torch.zeros(n, dtype=torch.float32, device="cuda")
+    out = torch.full((n,), -1, dtype=torch.int16, device="cuda")
+    for _ in range(3):                             # the first launch may still plan with a stale dealing offset
+        before = counts(lib)
+        lib.sideaware_one_to_one(kid, n * 4, out.data_ptr(), src.data_ptr(), 0, stream)
+        torch.cuda.synchronize()
+        assert counts(lib)[0] == before[0] + 1
+    xcd = out.view(-1, 8192 // 4)                  # one row per input granule (2048 elements)
+    assert bool((xcd == xcd[:, :1]).all()), "an input granule was handled by more than one XCD"
+    assert int(xcd.min()) >= 0 and int(xcd.max()) <= 7
+    half = (xcd[:, 0] // 4).cpu().tolist()
+    checked = 0
+    for g in range(0, len(half), 97):
+        side = lib.sideaware_side_of(src.data_ptr() + g * 8192)
+        assert side in (0, 1)
+        assert half[g] == side, (g, half[g], side)
+        checked += 1
+    assert checked > 50
     assert not sa.sideaware_last_error()
 
 
