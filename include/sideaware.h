@@ -215,9 +215,11 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * whose first output (first input, for an op whose output is narrower) lies in an arena of known sides use
  * the sided map, 0: never), "sided_min_bytes" (arrays
  * shorter than this never do), "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
- * -1: by array size) and "sided_wrong" (1: sided launches give every XCD the granules of the other half
+ * -1: by array size), "sided_wrong" (1: sided launches give every XCD the granules of the other half
  * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,
- * every access crossing between the dies).
+ * every access crossing between the dies) and "sided_widening" (1: an op whose every input is narrower
+ * than its output is sided too, following its first input; 0, the default: such ops use the striped map,
+ * which is as fast for them).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -98,20 +98,22 @@ struct SideMap {
 
 inline unsigned int parity32(unsigned int v) { return (unsigned int)__builtin_popcount(v) & 1u; }
 
-// True when a kernel whose tiles are tile_vectors * 16 bytes can run sided: a power-of-two number of
-// tiles per granule, an even number of XCDs.
-inline bool sided_tile_ok(int tile_vectors, int num_xcds) {
-    const uint64_t tile_bytes = (uint64_t)tile_vectors * 16;
+// True when a kernel whose tiles are tile_vectors * vector_bytes bytes of the array it follows can
+// run sided: a power-of-two number of tiles per granule, an even number of XCDs.
+inline bool sided_tile_ok(int tile_vectors, int num_xcds, unsigned int vector_bytes = 16) {
+    const uint64_t tile_bytes = (uint64_t)tile_vectors * vector_bytes;
     return tile_bytes >= 16 && tile_bytes <= (1u << kSideGranuleLog2) && (tile_bytes & (tile_bytes - 1)) == 0 &&
            num_xcds >= 2 && (num_xcds & (num_xcds - 1)) == 0;
 }
 
-// base_address must be a multiple of the tile size (the caller checks); stripe_pairs_log2 is r.
+// base_address is that of the array the launch follows and must be a multiple of the tile size (the
+// caller checks); vector_bytes is what one vector of the kernel covers of that array (16 unless the
+// array is narrower than the widest one); stripe_pairs_log2 is r.
 inline LaunchPlan plan_launch_sided(uint64_t base_address, long long num_vectors, int tile_vectors, int num_xcds,
                                     unsigned int stripe_pairs_log2, long long slot_run, long long slots_wanted,
-                                    const SideMap& side) {
+                                    const SideMap& side, unsigned int vector_bytes = 16) {
     LaunchPlan p;
-    const uint64_t tile_bytes = (uint64_t)tile_vectors * 16;
+    const uint64_t tile_bytes = (uint64_t)tile_vectors * vector_bytes;
     unsigned int tpg_log2 = 0;                                   // log2(tiles per granule)
     while ((tile_bytes << (tpg_log2 + 1)) <= (1u << kSideGranuleLog2)) tpg_log2++;
     const long long half = num_xcds / 2;                         // XCDs per side

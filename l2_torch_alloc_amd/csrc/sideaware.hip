@@ -95,22 +95,23 @@ struct Tuning {
     long long sided_min_bytes = 8ll << 20;   // ... when the array is at least this long
     long long sided_stripe = -1;     // log2(pairs per stripe of an XCD) of the sided map; -1: by array size
     long long sided_wrong = 0;       // 1: sided launches give every XCD the granules of the *other* half (an A/B switch)
+    long long sided_widening = 0;    // 1: ops whose every input is narrower than the output are sided too, following i0 (an A/B switch)
 };
 
 // The knobs themselves: written by sideaware_tune (and once from the environment), read by every
 // launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
 // a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
-constexpr int kTuneKnobs = 13;
+constexpr int kTuneKnobs = 14;
 static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
                                                    "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd",
                                                    "write_through", "sided", "sided_min_bytes", "sided_stripe",
-                                                   "sided_wrong"};
+                                                   "sided_wrong", "sided_widening"};
 static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
                                                  "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
                                                  "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD",
                                                  "SIDEAWARE_WRITE_THROUGH", "SIDEAWARE_SIDED", "SIDEAWARE_SIDED_MIN_BYTES",
-                                                 "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG"};
-static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}};
+                                                 "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG", "SIDEAWARE_SIDED_WIDENING"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}, {0}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -141,6 +142,7 @@ static Tuning tuning_snapshot() {
     t.sided_min_bytes = g_tune[10].load(std::memory_order_relaxed);
     t.sided_stripe = g_tune[11].load(std::memory_order_relaxed);
     t.sided_wrong = g_tune[12].load(std::memory_order_relaxed);
+    t.sided_widening = g_tune[13].load(std::memory_order_relaxed);
     return t;
 }
 
@@ -418,7 +420,8 @@ struct CompiledKernel {
     int vgprs = 0, sgprs = 0;
     int occupancy = 0;          // workgroups per CU the hardware can hold
     int tile_vectors = 0;       // from the module's sideaware_kernel_meta
-    int owner_is_o0 = 0;
+    int owner_is_o0 = 0;        // the array whose address decides ownership: o0 (1) or i0 (0)
+    int vec_size = 0;           // elements per vector
     bool sided = false;         // built with the sided ownership map
     bool gathered = false;      // inputs 1..3 go through the op's own indexing()
     unsigned char in_size[4] = {0, 0, 0, 0}, out_size[4] = {0, 0, 0, 0};   // element bytes per slot, 0: unused
@@ -559,6 +562,7 @@ static const CompiledKernel* build_kernel(DeviceContext* ctx, int kernel_id, Ker
         if (n > 1 && name[0]) e.function_name = name;                 // e.mu is held
         k.tile_vectors = meta[0];
         k.owner_is_o0 = meta[2];
+        k.vec_size = meta[1];
         k.sided = (meta[5] & 1) != 0;
         k.gathered = (meta[5] & 2) != 0;
         for (int j = 0; j < 4; j++) {
@@ -730,10 +734,18 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
     return false;
 }
 
+// What one vector of the kernel covers of the array a sided launch follows: 16 bytes unless that
+// array is narrower than the widest one (an op that only widens follows its narrower input).
+static unsigned int followed_vector_bytes(const CompiledKernel* k) {
+    const int size = k->owner_is_o0 ? k->out_size[0] : k->in_size[0];
+    const int bytes = k->vec_size * size;
+    return bytes > 0 && bytes <= 16 ? (unsigned int)bytes : 16u;
+}
+
 // Whether this launch of the sided instantiation `k` may go ahead, and with which arena constants.
-// A sided launch follows one array, the wider of o0 and i0 (o0 when they are as wide as each other;
-// num_bytes is that array's length): it must lie in an arena whose sides were measured and start on
-// a granule boundary.  Every other array that is as wide and accessed at the same index (outputs;
+// A sided launch follows one array (the kernel template says which: o0 for an op whose i0 is as wide,
+// i0 for one that narrows or only widens; num_bytes is the length of the widest array): it must lie in
+// an arena whose sides were measured and start on a granule boundary.  Every other array that is as wide and accessed at the same index (outputs;
 // inputs unless gathered through a custom `indexing`) is then on the right half of the device
 // wherever its side pattern matches the followed array's, and on the wrong half wherever it does not
 // (every access crossing between the dies).  Measured with a 256 MiB copy: all matching 6.9 TB/s, none
@@ -747,7 +759,8 @@ static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const v
     const void* owner = k->owner_is_o0 ? out[0] : in[0];
     const int owner_size = k->owner_is_o0 ? k->out_size[0] : k->in_size[0];
     if (owner == nullptr || owner_size == 0 || ((uintptr_t)owner & ((1u << kSideGranuleLog2) - 1)) != 0) return false;
-    if (!sides.lookup(owner, num_bytes, map)) return false;
+    const size_t owner_bytes = num_bytes / 16 * followed_vector_bytes(k);
+    if (!sides.lookup(owner, owner_bytes, map)) return false;
     const SideHash hash = sides.hash();
     uintptr_t owner_base = 0;
     unsigned int owner_flip = 0;
@@ -760,20 +773,16 @@ static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const v
         constexpr int kSamples = 64;
         int agree = 0;
         for (int i = 0; i < kSamples; i++) {
-            const uint64_t off = (uint64_t)(num_bytes / kSamples) * (unsigned)i;
+            const uint64_t off = (uint64_t)(owner_bytes / kSamples) * (unsigned)i;
             const unsigned int a = side_parity(((uintptr_t)p - base + off) & hash.address_mask) ^ flip;
             const unsigned int b = side_parity(((uintptr_t)owner - owner_base + off) & hash.address_mask) ^ owner_flip;
             agree += a == b;
         }
         return agree * 10 >= kSamples * 7;
     };
-    bool any_input = false, any_as_wide = false;
     for (int j = 0; j < 4; j++) {
-        if (!in[j] || k->in_size[j] == 0) continue;
+        if (!in[j] || k->in_size[j] != owner_size) continue;
         if (j > 0 && k->gathered) continue;
-        any_input = true;
-        if (k->in_size[j] != owner_size) continue;
-        any_as_wide = true;
         if (!follows(in[j])) return false;
     }
     for (int j = 0; j < 4; j++) {
@@ -781,9 +790,11 @@ static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const v
         if (!follows(out[j])) return false;
     }
     // An op that only widens (every input narrower than the output: an MXFP8 -> bf16 dequantise)
-    // loses with the sided map, 6.1 against 6.4 TB/s: the halves of each of its input granules go to
-    // XCDs of different sides.  An op with no input at all (a fill) only gains.
-    if (any_input && !any_as_wide) return false;
+    // would follow its input, but gains nothing from it: two thirds of its traffic are stores, half of
+    // which still cross (256 MiB out, nothing cache-resident: 6.39 TB/s against 6.44 striped; following
+    // the output instead, which splits every input granule between the sides, 6.13).  It stays on the
+    // striped map unless the switch says otherwise.
+    if (!k->owner_is_o0 && k->in_size[0] < k->out_size[0] && !t.sided_widening) return false;
     // The counterpart of the reference's FORCE_WRONG_SIDE (sideaware.cu:70-75, 297-298): the same
     // map with the arena's constant inverted, so that every access crosses to the other half.
     if (t.sided_wrong) map->flip ^= 1u;
@@ -947,7 +958,8 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     if (k->sided) {
         feedback = ctx->backing->sides().feedback_slot(stream, &side.dealing);
         plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0), num_vectors, k->tile_vectors,
-                                 ctx->num_xcds, sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side);
+                                 ctx->num_xcds, sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side,
+                                 followed_vector_bytes(k));
     } else {
         const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0);
         plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,
@@ -1066,7 +1078,8 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
                 sides[i].dealing = dealing;
                 plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]), num_vectors,
                                          k->tile_vectors, ctx->num_xcds,
-                                         sided_stripe_for(g.num_bytes, g.out[0] == g.in[0], t), t.slot_run, slots_wanted, sides[i]);
+                                         sided_stripe_for(g.num_bytes, g.out[0] == g.in[0], t), t.slot_run, slots_wanted, sides[i],
+                                         followed_vector_bytes(k));
             } else {
                 const uint64_t base = (uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]);
                 plan = plan_launch(base, num_vectors, k->tile_vectors, ctx->num_xcds,

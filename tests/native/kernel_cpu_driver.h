@@ -14,6 +14,8 @@
 //   addressed with the same element index and that element_idx counts elements of the array.
 // SA_CASE_NARROW: float in, short out: the input is the wider array, so ownership (striped or sided)
 //   follows i0's address.
+// SA_CASE_WIDEN: short in, float out: striped ownership follows o0, the sided map the narrower i0
+//   (tiles of half as many bytes).
 #include <cstdio>
 #include <cstdlib>
 
@@ -32,7 +34,7 @@ static sideaware::LaunchPlan make_plan(unsigned long long base, long long nv, un
         side.flip = (unsigned)(nv & 1);
         side.dealing = (unsigned)((grid + nv + g_stripe_log2) % SA_NUM_XCD);
         return sideaware::plan_launch_sided(base, nv, sideaware_kernel_meta[0], SA_NUM_XCD, g_stripe_log2 % 9,
-                                            g_slot_run, grid / SA_NUM_XCD, side);
+                                            g_slot_run, grid / SA_NUM_XCD, side, (unsigned)sa_followed_vector_bytes);
     }
     return sideaware::plan_launch(base, nv, sideaware_kernel_meta[0], SA_NUM_XCD,
                                   1ull << g_stripe_log2, g_slot_run, grid / SA_NUM_XCD);
@@ -164,6 +166,21 @@ static int run_case(unsigned grid, long long nv, size_t off) {
     for (size_t i = 0; i < n; i++) bad += (((short*)s_out.data)[i] != (short)(i % 3001) + 1);
     return bad;
 }
+#elif defined(SA_CASE_WIDEN)
+static int run_case(unsigned grid, long long nv, size_t off) {
+    const size_t n = (size_t)nv * vec_size;
+    // o0 is the wider array (shifted by `off`); the only input is narrower, and a sided instantiation
+    // follows it: half a tile of o0's bytes per tile
+    Arena f_out(off, n * sizeof(float)), s_in(off / 2, n * sizeof(short));
+    short* si = (short*)s_in.data;
+    for (size_t i = 0; i < n; i++) si[i] = (short)(i % 3001);
+    std::memset(f_out.data, 0xff, n * sizeof(float));
+    run_grid(grid, (size_type)nv, (vo0*)f_out.data, nullptr, nullptr, nullptr, (const vi0*)si, nullptr, nullptr, nullptr,
+             nullptr, 0);
+    int bad = !f_out.sentinel_ok() + !s_in.sentinel_ok();
+    for (size_t i = 0; i < n; i++) bad += (((float*)f_out.data)[i] != (float)(i % 3001) + 0.5f);
+    return bad;
+}
 #elif defined(SA_CASE_ROPE)
 // The op header under test is a generated RoPE header; rope_T / rope_half / rope_heads /
 // rope_rotated come from it.  The activation holds `nv` vectors (any length: a whole number of
@@ -210,7 +227,7 @@ static int run_case(unsigned grid, long long nv, size_t off) {
     return bad;
 }
 #else
-#error "define SA_CASE_INCREMENT, SA_CASE_MIXED, SA_CASE_NARROW or SA_CASE_ROPE"
+#error "define SA_CASE_INCREMENT, SA_CASE_MIXED, SA_CASE_NARROW, SA_CASE_WIDEN or SA_CASE_ROPE"
 #endif
 
 int main() {

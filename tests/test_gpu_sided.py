@@ -67,7 +67,8 @@ def lib(sa):
     if L.sideaware_side_address_mask() == 0:
         pytest.skip("the device showed no side structure to the start-up probe")
     yield L
-    for key, value in ((b"sided", 1), (b"sided_wrong", 0), (b"sided_stripe", -1), (b"sided_min_bytes", 8 * MiB)):
+    for key, value in ((b"sided", 1), (b"sided_wrong", 0), (b"sided_stripe", -1), (b"sided_min_bytes", 8 * MiB),
+                       (b"sided_widening", 0)):
         assert L.sideaware_tune(key, value) == 0
 
 
@@ -292,6 +293,60 @@ def test_a_narrowing_op_runs_on_the_side_of_its_input(sa, lib):
         assert half[g] == side, (g, half[g], side)
         checked += 1
     assert checked > 50
+    assert not sa.sideaware_last_error()
+
+
+def test_a_widening_op_is_striped_unless_asked_and_then_follows_its_input(sa, lib):
+    """short in, int out (every input narrower than the output): striped by default, which is as
+    fast for such ops; with the `sided_widening` switch the sided map follows the input, so each
+    8 KiB input granule and the 16 KiB of output it becomes are handled by one XCD of the half of
+    the device that holds the input granule."""
+    stream = torch.cuda.current_stream().cuda_stream
+    kid = sa.sideaware_create_kernel(b"""
+#define KERNEL_NAME sideaware_test_widening_xcd_id
+typedef int o0;
+typedef short i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
+                                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    out0 = (int)(xcc & 0xf) + 1000 * (int)in0;
+}
+""")
+    n = 16 * MiB                                   # elements: 32 MiB in, 64 MiB out
+    src = torch.randint(0, 100, (n,), dtype=torch.int16, device="cuda")
+    out = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    before = counts(lib)
+    lib.sideaware_one_to_one(kid, n * 4, out.data_ptr(), src.data_ptr(), 0, stream)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0], before[1] + 1)
+    assert torch.equal(out // 1000, src.int())
+    assert lib.sideaware_tune(b"sided_widening", 1) == 0
+    try:
+        for _ in range(3):                         # the first launch may still plan with a stale dealing offset
+            out.fill_(-1)
+            before = counts(lib)
+            lib.sideaware_one_to_one(kid, n * 4, out.data_ptr(), src.data_ptr(), 0, stream)
+            torch.cuda.synchronize()
+            assert counts(lib) == (before[0] + 1, before[1])
+    finally:
+        assert lib.sideaware_tune(b"sided_widening", 0) == 0
+    assert torch.equal(out // 1000, src.int())
+    xcd = (out % 1000).view(-1, 8192 // 2)         # one row per input granule (4096 elements)
+    assert bool((xcd == xcd[:, :1]).all()), "an input granule was handled by more than one XCD"
+    half = (xcd[:, 0] // 4).cpu().tolist()
+    checked = 0
+    for g in range(0, len(half), 97):
+        side = lib.sideaware_side_of(src.data_ptr() + g * 8192)
+        assert side in (0, 1)
+        assert half[g] == side, (g, half[g], side)
+        checked += 1
+    assert checked > 40
     assert not sa.sideaware_last_error()
 
 

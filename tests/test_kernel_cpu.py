@@ -71,6 +71,21 @@ __device__ void elementwise_op(size_t element_idx, int sideband,
 }
 """
 
+WIDEN_HEADER = """
+typedef float o0;
+typedef short i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = %(reverse)s;
+constexpr bool input_evict[4] = {true, false, false, false};
+%(unrolled)s
+__device__ void elementwise_op(size_t element_idx, int sideband,
+                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = (float)in0 + 0.5f;
+}
+"""
+
 
 @pytest.fixture(scope="module")
 def lib():
@@ -87,7 +102,7 @@ def build_driver(lib, tmp_path, case, variant, unrolled, reverse, header=None):
     config = lib.sideaware_config_block(variant).decode()
     template = lib.sideaware_kernel_source().decode()
     if header is None:
-        header = {"INCREMENT": INCREMENT_HEADER, "MIXED": MIXED_HEADER, "NARROW": NARROW_HEADER}[case] % {
+        header = {"INCREMENT": INCREMENT_HEADER, "MIXED": MIXED_HEADER, "NARROW": NARROW_HEADER, "WIDEN": WIDEN_HEADER}[case] % {
             "reverse": "true" if reverse else "false",
             "unrolled": "" if unrolled is None else "#define UNROLLED %d" % unrolled,
         }
@@ -141,11 +156,14 @@ CONFIGS = [
     ("INCREMENT", 33, 2, True),
     ("INCREMENT", 32, 2, False),
     ("INCREMENT", 33, 1, True),
-    ("MIXED", 32, 1, False),         # o0 is wider than i0: the map follows o0
+    ("MIXED", 32, 1, False),         # o0 is wider than i0 but as wide as i1: the map follows o0
     ("INCREMENT", 32, 4, False),     # tiles of 16 KiB cannot be sided: the instantiation falls back to stripes
     ("NARROW", 0, None, False),      # i0 is wider than o0: stripes follow i0
     ("NARROW", 32, 1, False),        # ... and so does the sided map
     ("NARROW", 33, 2, True),
+    ("WIDEN", 0, None, False),       # every input narrower than o0: stripes follow o0 ...
+    ("WIDEN", 32, 1, False),         # ... the sided map follows i0, whose tiles are 2 KiB here
+    ("WIDEN", 33, 4, True),          # and 8 KiB here (16 KiB of o0)
 ]
 
 
@@ -156,7 +174,7 @@ def test_template_on_cpu(lib, tmp_path, case, variant, unrolled, reverse):
     exe = build_driver(lib, tmp_path, case, variant, unrolled, reverse)
     rng = random.Random(hash((case, variant, unrolled, reverse)) & 0xffff)
     cases = cases_for(variant, unrolled, rng)
-    if case in ("MIXED", "NARROW"):
+    if case in ("MIXED", "NARROW", "WIDEN"):
         cases = [(g, n, off - off % 64, s, r) for (g, n, off, s, r) in cases]   # halved offsets stay 16 B-aligned
         lines = ["%d %d %d %d %d\n" % c for c in cases]
     else:
