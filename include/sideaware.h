@@ -172,6 +172,19 @@ int sideaware_xcd_dealing_verified(void);
  * Returns 0, or a HIP error code after recording a message for sideaware_last_error. */
 int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
                           int device, sideaware_stream_t stream);
+/* Makes device memory the pool did not hand out known to the sided map (no counterpart in the
+ * reference, whose side tables cover its own allocator's pages only): measures the constant of
+ * [region, region + num_bytes) as for an arena of the pool, after which launches over arrays inside it
+ * may use the sided map and sideaware_side_of answers for it.  The region must be one physically
+ * contiguous allocation (a single hipMalloc of the size this library's arenas have is; the vote over
+ * its granules says no otherwise), start on a multiple of 16 KiB, hold at least 128 MiB and overlap no
+ * region already known.  Waits for the measurement (a fraction of a millisecond).
+ * Returns 1 when the region's sides are known afterwards, 0 when they are not (it does not fit the
+ * hash, overlaps, the device was too busy to tell, or side probing is off), -1 for a bad argument
+ * (message in sideaware_last_error).  Unregister before freeing the memory; stale knowledge costs
+ * speed, never results. */
+int sideaware_register_region(void* region, size_t num_bytes, int device);
+void sideaware_unregister_region(void* region, int device);
 /* The same measurement for callers that cannot allocate (code under stream capture, tight serving
  * loops, harnesses that forbid it): no counterpart in the reference.  It allocates nothing and
  * frees nothing; its work space is a static device array of 32 KiB that every device the library

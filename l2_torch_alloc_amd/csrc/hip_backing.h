@@ -21,6 +21,11 @@ public:
 
     // What was measured about the arenas handed to the pool (side_map.h).
     SideRegistry& sides() { return sides_; }
+    // True when ptr is the start of an arena this backing store acquired and still holds.
+    bool owns_arena(void* ptr) {
+        std::lock_guard<std::mutex> lk(mu_);
+        return raw_of_.count(ptr) != 0;
+    }
 
 private:
     int device_;

@@ -101,8 +101,11 @@ public:
     explicit SideRegistry(int device) : device_(device) {}
     ~SideRegistry();
 
-    // Called by the backing store around hipMalloc / hipFree of an arena.
-    void add_arena(void* base, size_t bytes);
+    // Called by the backing store around hipMalloc / hipFree of an arena, and for memory a caller
+    // registers: measures the region's constant.  True when it is known afterwards; false when the
+    // samples do not fit the hash, the device was too busy to tell (a later placement tries again),
+    // or the region overlaps one already known (then nothing is recorded).
+    bool add_arena(void* base, size_t bytes);
     void remove_arena(void* base);
 
     // Measures the hash (once; add_arena does it too if nobody has).

@@ -445,14 +445,18 @@ void SideRegistry::vote_locked(ArenaSide& a) {
     }
 }
 
-void SideRegistry::add_arena(void* base, size_t bytes) {
+bool SideRegistry::add_arena(void* base, size_t bytes) {
     std::lock_guard<std::mutex> g(mu_);
     discover_locked();
     ArenaSide a;
     a.base = (uintptr_t)base;
     a.bytes = bytes;
+    for (const ArenaSide& other : arenas_) {
+        if (a.base < other.base + other.bytes && other.base < a.base + a.bytes) return false;   // overlaps a known one
+    }
     vote_locked(a);
     arenas_.push_back(a);
+    return a.known;
 }
 
 // An arena whose vote was inconclusive is measured again when the pool next places a region in

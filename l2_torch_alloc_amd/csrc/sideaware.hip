@@ -1266,6 +1266,32 @@ int sideaware_probe_sides_noalloc(const void* region, size_t num_bytes, unsigned
     return probe_sides_common("probe_sides_noalloc", region, num_bytes, seed, count, sides, device, stream, /*allocate=*/false);
 }
 
+int sideaware_register_region(void* region, size_t num_bytes, int device) {
+    DeviceContext* ctx = get_context(device);
+    if (!ctx) return -1;
+    if (!region || ((uintptr_t)region & ((1u << kSidePairLog2) - 1)) != 0 || num_bytes < (128u << 20)) {
+        set_error("register_region: region (%p) must start on a multiple of 16 KiB and hold at least 128 MiB (%zu)", region,
+                  num_bytes);
+        return -1;
+    }
+    hipPointerAttribute_t attr;
+    ScopedDevice guard(ctx->device);
+    if (hipPointerGetAttributes(&attr, region) != hipSuccess || attr.type != hipMemoryTypeDevice || attr.device != ctx->device) {
+        (void)hipGetLastError();
+        set_error("register_region: %p is not memory of device %d", region, ctx->device);
+        return -1;
+    }
+    return ctx->backing->sides().add_arena(region, num_bytes & ~(size_t)((1u << kSidePairLog2) - 1)) ? 1 : 0;
+}
+
+void sideaware_unregister_region(void* region, int device) {
+    DeviceContext* ctx = get_context(device);
+    if (!ctx || !region) return;
+    // never one of the pool's own arenas: those go when the pool gives them back
+    if (ctx->backing->owns_arena(region)) return;
+    ctx->backing->sides().remove_arena(region);
+}
+
 void sideaware_launch_counts(unsigned long long* sided, unsigned long long* striped) {
     if (sided) *sided = g_launches_sided.load(std::memory_order_relaxed);
     if (striped) *striped = g_launches_striped.load(std::memory_order_relaxed);

@@ -73,6 +73,8 @@ _SIGNATURES = {
     "sideaware_xcd_dealing_verified": (_ci, []),
     "sideaware_probe_sides": (_ci, [_vp, _sz, ctypes.c_ulonglong, _ci, _vp, _ci, _vp]),
     "sideaware_probe_sides_noalloc": (_ci, [_vp, _sz, ctypes.c_ulonglong, _ci, _vp, _ci, _vp]),
+    "sideaware_register_region": (_ci, [_vp, _sz, _ci]),
+    "sideaware_unregister_region": (None, [_vp, _ci]),
     "sideaware_side_address_mask": (ctypes.c_ulonglong, []),
     "sideaware_side_of": (_ci, [_vp]),
     "sideaware_stream_dealing": (_ci, [_vp]),

@@ -51,6 +51,21 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
 }
 """
 
+ADD_ONE_HEADER = b"""
+#define KERNEL_NAME sideaware_test_add_one
+typedef unsigned char o0;
+typedef unsigned char i0;
+struct unused {};
+typedef unused o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
+                                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {
+    out0 = (unsigned char)(in0 + 1);
+}
+"""
+
 
 def counts(lib):
     a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
@@ -347,6 +362,74 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
         assert half[g] == side, (g, half[g], side)
         checked += 1
     assert checked > 40
+    assert not sa.sideaware_last_error()
+
+
+def test_registered_foreign_memory_gets_sided_launches(sa, lib):
+    """Memory straight from hipMalloc is unknown to the pool: launches over it are striped and
+    sideaware_side_of says -1.  Once registered, its sides are measured like an arena's: side_of
+    answers (and agrees with a fresh probe), an in-place launch over it is sided, and results stay
+    bit-exact.  Unregistered, it is unknown again."""
+    stream = torch.cuda.current_stream().cuda_stream
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+    hip.hipMalloc.restype = ctypes.c_int
+    hip.hipFree.argtypes = [ctypes.c_void_p]
+    hip.hipFree.restype = ctypes.c_int
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    hip.hipMemcpy.restype = ctypes.c_int
+    n = 256 * MiB
+    raw = ctypes.c_void_p()
+    assert hip.hipMalloc(ctypes.byref(raw), n) == 0 and raw.value
+    try:
+        base = raw.value
+        assert base % 16384 == 0
+        seed = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+        back = torch.empty_like(seed)
+        assert hip.hipMemcpy(base, seed.data_ptr(), n, 3) == 0               # device to device
+        kid = sa.sideaware_create_kernel(ADD_ONE_HEADER)
+
+        def add_one_in_place():
+            before = counts(lib)
+            lib.sideaware_one_to_one(kid, n, base, base, 0, stream)
+            torch.cuda.synchronize()
+            after = counts(lib)
+            return after[0] - before[0], after[1] - before[1]
+
+        assert lib.sideaware_side_of(base) == -1
+        assert add_one_in_place() == (0, 1)
+        assert lib.sideaware_register_region(base + 4096, n - 4096, 0) == -1      # not on a 16 KiB boundary
+        assert "16 KiB" in sa.sideaware_last_error()
+        lib.sideaware_clear_error()
+        known = lib.sideaware_register_region(base, n, 0)
+        assert known in (0, 1)
+        if known == 0:
+            pytest.skip("this allocation's sides did not fit the hash (not one physically contiguous run)")
+        assert lib.sideaware_register_region(base, n, 0) == 0                     # overlaps what is known
+        assert lib.sideaware_side_of(base) in (0, 1)
+        assert lib.sideaware_side_of(base) != lib.sideaware_side_of(base + 8192)
+        count = 128
+        sides = torch.full((count,), -2, dtype=torch.int32, device="cuda")
+        assert lib.sideaware_probe_sides(base, n, 99, count, sides.data_ptr(), 0, stream) == 0
+        torch.cuda.synchronize()
+        granules = n // 8192
+        disagree = 0
+        for i, s_i in enumerate(sides.cpu().tolist()):
+            g = splitmix64(99 + i) % granules
+            if s_i >= 0:
+                disagree += s_i != lib.sideaware_side_of(base + g * 8192)
+        assert disagree <= count // 32
+        assert add_one_in_place() == (1, 0)
+        assert add_one_in_place() == (1, 0)
+        lib.sideaware_unregister_region(base, 0)
+        assert lib.sideaware_side_of(base) == -1
+        assert add_one_in_place() == (0, 1)
+        assert hip.hipMemcpy(back.data_ptr(), base, n, 3) == 0
+        assert torch.equal(back, seed + 4)                                         # uint8 arithmetic wraps
+    finally:
+        lib.sideaware_unregister_region(raw, 0)
+        torch.cuda.synchronize()
+        assert hip.hipFree(raw) == 0
     assert not sa.sideaware_last_error()
 
 
