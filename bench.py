@@ -211,6 +211,81 @@ def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4, named_kernels=F
     return out
 
 
+# Reads its input and writes nothing (a scan that would report through the sideband pointer): the
+# condition keeps the loads alive and is false for the data used here.
+READ_ONLY_HEADER = b"""
+#define KERNEL_NAME sideaware_bench_read_only
+typedef int i0;
+struct unused {};
+typedef unused o0, o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
+                                               o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}
+#define CUSTOM_VECTOR_OP
+__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size,
+                          o0 *out0, o1 *out1, o2 *out2, o3 *out3,
+                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,
+                          int* sideband_memory, int sideband_value) {
+    if ((in0[0] ^ in0[1] ^ in0[2] ^ in0[3]) == sideband_value) sideband_memory[0] = 1;
+}
+"""
+
+
+def bench_one_direction(nbytes=GiB, sets=4, steps=12, rounds=3):
+    """What the memory system gives the library's kernels in one direction only, buffers cycling
+    so that nothing is cache-resident: a fill (stores only) and a scan (loads only), each with the
+    sided and with the XCD-striped map in turn (medians).  The copy's own ceiling is the harmonic
+    mix of the two."""
+    import torch
+    from l2_torch_alloc_amd import headers, wrapper
+    lib, stream = _abi()
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    hit = torch.zeros(4, dtype=torch.int32, device="cuda")
+    kid_fill = wrapper.sideaware_create_kernel(headers.fill_header())
+    kid_scan = wrapper.sideaware_create_kernel(READ_ONLY_HEADER)
+    counter = [0]
+
+    def fill():
+        i = counter[0] % sets
+        counter[0] += 1
+        lib.sideaware_elementwise(kid_fill, nbytes, bufs[i].data_ptr(), 0, 0, 0, 0, 0, 0, 0, 0, 0x01010101 * (1 + i), 0, 0, 0, stream)
+
+    def scan(needle=0x5bd1e995):
+        i = counter[0] % sets
+        counter[0] += 1
+        lib.sideaware_elementwise(kid_scan, nbytes, 0, 0, 0, 0, bufs[i].data_ptr(), 0, 0, 0, hit.data_ptr(), needle, 0, 0, 0, stream)
+
+    for _ in range(sets):
+        fill()
+    cases = {"scan": scan, "fill": fill}
+    times = {(name, sided): [] for name in cases for sided in (1, 0)}
+    try:
+        for _ in range(rounds):
+            for name, fn in cases.items():
+                for sided in (1, 0):
+                    lib.sideaware_tune(b"sided", sided)
+                    times[(name, sided)].append(time_region(fn, steps, sets))
+    finally:
+        lib.sideaware_tune(b"sided", 1)
+    torch.cuda.synchronize()
+    # the fills wrote what they were told to, the scans found no needle; a scan for a value that is
+    # there (the xor of four equal words is 0) does report
+    ok = all(bool((b.view(torch.int32)[::4097] == 0x01010101 * (1 + i)).all()) for i, b in enumerate(bufs))
+    ok = ok and int(hit[0]) == 0
+    scan(needle=0)
+    torch.cuda.synchronize()
+    ok = ok and int(hit[0]) == 1
+    out = {"bytes": nbytes, "sets": sets, "results_ok": ok}
+    for name in cases:
+        for sided in (1, 0):
+            sec = statistics.median(times[(name, sided)])
+            out["%s_%s" % (name, "sided" if sided else "xcd_striped")] = {
+                "us": sec * 1e6, "GBps": gbps(nbytes, sec), "frac_of_peak": gbps(nbytes, sec) / HBM_PEAK_GBPS}
+    return out
+
+
 def bench_vendor_copies(nbytes, pairs, steps):
     """The same cycling copy done by the platform's own copy paths, for scale: PyTorch's copy_
     kernel and the runtime's device-to-device hipMemcpyAsync, on the same kind of buffers."""
@@ -853,6 +928,8 @@ def main():
         also["copy_sweep"] = sweep
         also["copy_256MiB_ownership_map_ab"] = bench_side_ab()
         log("ownership map A/B:", also["copy_256MiB_ownership_map_ab"])
+        also["one_direction_1GiB"] = bench_one_direction()
+        log("one direction only:", also["one_direction_1GiB"])
         also["copy_4MiB_replayed_from_a_hip_graph"] = bench_small_copy_in_graph()
         log("graph:", also["copy_4MiB_replayed_from_a_hip_graph"])
         also["energy_copy_1GiB"] = bench_energy()

@@ -160,6 +160,30 @@ __device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband,
     ops.fill_int32(z, 7)
     torch.cuda.synchronize()
     assert counts(lib) == (before[0] + 1, before[1]) and bool((z == 7).all())
+    # an op with no output at all (a scan that reports through the sideband pointer) follows its input
+    scan = sa.sideaware_create_kernel(b"""
+#define KERNEL_NAME sideaware_test_scan
+typedef int i0;
+struct unused {};
+typedef unused o0, o1, o2, o3, i1, i2, i3;
+constexpr bool reverse_order = false;
+constexpr bool input_evict[4] = {true, false, false, false};
+__device__ __forceinline__ void elementwise_op(size_t element_idx, int sideband, o0 &out0, o1 &out1, o2 &out2, o3 &out3,
+                                               const i0 &in0, const i1 &in1, const i2 &in2, const i3 &in3) {}
+#define CUSTOM_VECTOR_OP
+__device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *out0, o1 *out1, o2 *out2, o3 *out3,
+                                          const i0 *in0, const i1 *in1, const i2 *in2, const i3 *in3,
+                                          int* sideband_memory, int sideband_value) {
+    for (int i = 0; i < 4; i++) if (in0[i] == sideband_value) atomicAdd(sideband_memory, 1);
+}
+""")
+    hits = torch.zeros(4, dtype=torch.int32, device="cuda")
+    z[12345] = 8
+    z[-1] = 8
+    before = counts(lib)
+    lib.sideaware_elementwise(scan, z.numel() * 4, 0, 0, 0, 0, z.data_ptr(), 0, 0, 0, hits.data_ptr(), 8, 0, 0, 0, stream)
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0] + 1, before[1]) and int(hits[0]) == 2
     # an op whose output is narrower than its input follows the input: the input must be in measured
     # memory and start on a granule boundary, the output may be anywhere
     narrow = sa.sideaware_create_kernel(NARROWING_XCD_ID_HEADER)
