@@ -836,6 +836,8 @@ def main():
     ap.add_argument("--side-ab", action="store_true",
                     help="only the 256 MiB copy under the three ownership maps (sided, XCD-striped, sided the wrong "
                          "way round), each under a kernel name of its own (for a kernel trace)")
+    ap.add_argument("--one-direction", action="store_true",
+                    help="only the 1 GiB scan (loads only) and fill (stores only) under the sided and the striped map")
     ap.add_argument("--only", action="append", default=None,
                     help="with an experiment mode: run only the cases whose name contains this text")
     ap.add_argument("--churn-baseline", action="store_true", help=argparse.SUPPRESS)
@@ -866,6 +868,9 @@ def main():
         import bench_experiments as experiments      # the sweep modes: not needed by the default run
     if args.side_ab:
         print(json.dumps({"copy_256MiB_ownership_map_ab": bench_side_ab(named_kernels=True)}))
+        return
+    if args.one_direction:
+        print(json.dumps({"one_direction_1GiB": bench_one_direction()}))
         return
     if args.stripe_ab:
         print(json.dumps({"stripe_ab": experiments.stripe_ab(args.steps)}))
