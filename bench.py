@@ -123,14 +123,19 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
     are those of the launches before it: the steady state of a streaming pipeline.  The first
     source holds the seeded values (uint8 uniform in [0, 255] from `seed`, made on the host), the
     others the same kind of values made on the device; every destination is compared with its
-    source afterwards."""
+    source afterwards.  Each destination is allocated right after its source, as a program that
+    makes an output for an input would: the pool then places the two so that their sides agree
+    over 99 % of their length (all sources first, then all destinations: 94 %, and 0.8 % less
+    throughput at 256 MiB)."""
     import torch
-    if nbytes <= GiB:
-        first = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=torch.Generator().manual_seed(seed)).cuda()
-    else:                                        # too long to make on the host in reasonable time
-        first = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
-    srcs = [first] + [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs - 1)]
-    dsts = [torch.zeros_like(t) for t in srcs]
+    srcs, dsts = [], []
+    for i in range(pairs):
+        if i == 0 and nbytes <= GiB:             # (longer ones take too long to make on the host)
+            src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=torch.Generator().manual_seed(seed)).cuda()
+        else:
+            src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+        srcs.append(src)
+        dsts.append(torch.zeros_like(src))
     lib, stream = _abi()
     ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
     counter = [0]
@@ -156,8 +161,10 @@ def bench_side_ab(nbytes=256 * MiB, pairs=8, steps=30, rounds=4, named_kernels=F
     sideaware.cu:70-75)."""
     import ctypes
     import torch
-    srcs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(pairs)]
-    dsts = [torch.zeros_like(t) for t in srcs]
+    srcs, dsts = [], []
+    for _ in range(pairs):                       # each destination right after its source, as in the headline
+        srcs.append(torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda"))
+        dsts.append(torch.zeros_like(srcs[-1]))
     lib, stream = _abi()
     ptrs = [(d.data_ptr(), t.data_ptr()) for d, t in zip(dsts, srcs)]
     counter = [0]
@@ -546,10 +553,14 @@ def bench_other_ops_cycling(steps, sets=4):
     from l2_torch_alloc_amd import headers, wrapper
     lib, stream = _abi()
     n = 256 * MiB // 2                                                     # bf16 elements
-    xs = [torch.randn(n, device="cuda").to(torch.bfloat16) for _ in range(sets)]
-    ys = [torch.empty_like(x) for x in xs]
-    qs = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(sets)]
-    ss = [torch.empty(n // 32, dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    xs, ys, qs, ss = [], [], [], []
+    for _ in range(sets):                        # one group after the other, outputs right after their input
+        x32 = torch.randn(n, device="cuda")
+        xs.append(x32.to(torch.bfloat16))
+        del x32
+        ys.append(torch.empty_like(xs[-1]))
+        qs.append(torch.empty(n, dtype=torch.uint8, device="cuda"))
+        ss.append(torch.empty(n // 32, dtype=torch.uint8, device="cuda"))
     sb = torch.tensor([1.25, -0.5], dtype=torch.float32, device="cuda")
     counter = [0]
 

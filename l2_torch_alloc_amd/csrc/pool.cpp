@@ -129,7 +129,9 @@ bool Pool::extent_take_locked(int kind, size_t bytes, uintptr_t* addr, Extent* t
             const uintptr_t at = backing_->place_canonical(cand->second, cand->second + cand->first, bytes, /*lines=*/true);
             if (at == 0) continue;
             assert(at >= cand->second && at + bytes <= cand->second + cand->first && at % kRegionAlign == 0);
-            if (at - cand->second > std::max<size_t>(kCanonicalSlack, bytes / kCanonicalGapDivisor)) continue;   // too large a hole in front
+            const size_t divisor = bytes <= kCanonicalSmallBytes ? kCanonicalGapDivisorSmall
+                                 : bytes <= 2 * kCanonicalSmallBytes ? kCanonicalGapDivisorMid : kCanonicalGapDivisor;
+            if (at - cand->second > std::max<size_t>(kCanonicalSlack, bytes / divisor)) continue;   // too large a hole in front
             sit = cand;
             start = at;
             placed = true;
