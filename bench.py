@@ -116,24 +116,29 @@ def bench_copy_cold(nbytes, steps):
             "after_read_scrub": {"us_median": clean * 1e6, "GBps": gbps(2 * nbytes, clean)}}
 
 
-def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
+def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0, dtype="uint8"):
     """The headline protocol.  `steps` back-to-back launches that cycle through `pairs` distinct
     (src, dst) pairs, so no launch finds an operand in a cache (the working set is
     pairs * 2 * nbytes, far beyond the 256 MB Infinity Cache) and the only dirty lines in its way
     are those of the launches before it: the steady state of a streaming pipeline.  The first
-    source holds the seeded values (uint8 uniform in [0, 255] from `seed`, made on the host), the
-    others the same kind of values made on the device; every destination is compared with its
+    source holds the seeded values (uint8 uniform in [0, 255], or fp32 uniform in (-1, 1) for the
+    size sweep, from `seed`, made on the host), the others the same kind of values made on the device; every destination is compared with its
     source afterwards.  Each destination is allocated right after its source, as a program that
     makes an output for an input would: the pool then places the two so that their sides agree
     over 99 % of their length (all sources first, then all destinations: 94 %, and 0.8 % less
     throughput at 256 MiB)."""
     import torch
     srcs, dsts = [], []
+    torch.cuda.manual_seed(seed)
     for i in range(pairs):
-        if i == 0 and nbytes <= GiB:             # (longer ones take too long to make on the host)
-            src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=torch.Generator().manual_seed(seed)).cuda()
-        else:
-            src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+        on_host = i == 0 and nbytes <= GiB       # (longer ones take too long to make on the host)
+        gen = torch.Generator().manual_seed(seed)
+        if dtype == "uint8":
+            src = (torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen).cuda() if on_host
+                   else torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda"))
+        else:                                    # fp32 uniform in (-1, 1): the sweep's values
+            src = ((torch.rand(nbytes // 4, generator=gen) * 2 - 1).cuda() if on_host
+                   else torch.empty(nbytes // 4, dtype=torch.float32, device="cuda").uniform_(-1, 1))
         srcs.append(src)
         dsts.append(torch.zeros_like(src))
     lib, stream = _abi()
@@ -149,7 +154,7 @@ def bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=0, prewarm=0):
         launch()                                 # rest brings the device to its steady clocks
     sec = time_region(launch, steps, warmup)
     ok = all(bool(torch.equal(d, t)) for d, t in zip(dsts, srcs))
-    return {"bytes": nbytes, "pairs": pairs, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec),
+    return {"bytes": nbytes, "pairs": pairs, "dtype": dtype, "us": sec * 1e6, "GBps": gbps(2 * nbytes, sec),
             "frac_of_peak": gbps(2 * nbytes, sec) / HBM_PEAK_GBPS, "bit_exact": ok}
 
 
@@ -935,7 +940,7 @@ def main():
         sweep = {}
         for label, nbytes, pairs, steps in (("4MiB", 4 * MiB, 128, 512), ("64MiB", 64 * MiB, 8, 96),
                                             ("256MiB", 256 * MiB, 8, 48), ("1GiB", GiB, 4, 20), ("8GiB", 8 * GiB, 2, 6)):
-            cycling = bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=3, prewarm=pairs)
+            cycling = bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=3, prewarm=pairs, dtype="fp32")
             one_pair = bench_copy(nbytes, steps, 3, "fp32", seed=3)
             sweep[label] = {"hbm_cycling_pairs": cycling, "one_pair_in_a_loop": one_pair,
                             "working_set_bytes_cycling": 2 * nbytes * pairs}
