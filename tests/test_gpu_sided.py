@@ -307,6 +307,40 @@ def test_sided_launches_replay_from_a_hip_graph(sa, lib):
     assert not sa.sideaware_last_error()
 
 
+def test_the_dealing_offset_survives_other_kernels_on_the_stream(sa, lib):
+    """The sided map plans with the XCD that workgroup 0 of the stream's last sided launch ran on.
+    That offset belongs to the queue, not to its history: kernels of other shapes in between (PyTorch's
+    own, with odd workgroup counts) do not move it, so no sided launch after the first is planned
+    with a stale offset."""
+    import random
+    stream = torch.cuda.current_stream().cuda_stream
+    kid = sa.sideaware_create_kernel(XCD_ID_HEADER)
+    n = 32 * MiB
+    src = torch.zeros(n // 4, dtype=torch.int32, device="cuda")
+    out = torch.full((n // 4,), -1, dtype=torch.int32, device="cuda")
+    sides = torch.tensor([lib.sideaware_side_of(out.data_ptr() + g * 8192) for g in range(0, n // 8192, 61)], device="cuda")
+    assert int(sides.min()) >= 0
+
+    def launch():
+        out.fill_(-1)
+        believed = lib.sideaware_stream_dealing(stream)
+        lib.sideaware_one_to_one(kid, n, out.data_ptr(), src.data_ptr(), 0, stream)
+        torch.cuda.synchronize()
+        wrong = int(((out.view(-1, 2048)[::61, 0] // 4) != sides).sum())
+        return believed, lib.sideaware_stream_dealing(stream), wrong
+
+    for _ in range(2):
+        launch()
+    rng = random.Random(1)
+    for trial in range(12):
+        for _ in range(rng.randrange(1, 5)):
+            m = rng.choice([1, 3, 7, 100, 257, 4099, 65537]) * rng.choice([1, 64, 256])
+            a = torch.empty(m, device="cuda").normal_()
+            (a * 2 + 1).sum()
+        believed, reported, wrong = launch()
+        assert believed == reported and wrong == 0, (trial, believed, reported, wrong)
+
+
 def test_a_narrowing_op_runs_on_the_side_of_its_input(sa, lib):
     """float in, short out: the sided map follows the input (the wider array, two thirds of the
     traffic).  Every 8 KiB granule of the input is read, and its 4 KiB of output written, by an XCD
