@@ -37,7 +37,7 @@ from bench_util import GiB, HBM_PEAK_GBPS, MiB, _abi, gbps, log, time_each, time
 # 262144 KiB fetched, so x1.99983; WRITE_SIZE reads 262144.0, so x1.0).
 TRAFFIC_PROFILE = "profiles/sideaware_copy_256MiB_and_rope_bf16_llama3_hbm_traffic.txt"
 COPY_256MIB_TRAFFIC_BYTES = int((131084.1 * 1.99983 + 262144.0) * 1024)       # 536.9 MB, 1.0000 x algorithmic
-ROPE_STEP_TRAFFIC_BYTES = int((165813.5 * 1.99983 + 327680.0) * 1024)         # 675.1 MB, 1.0028 x algorithmic (q and k in one launch)
+ROPE_STEP_TRAFFIC_BYTES = int((165969.8 * 1.99983 + 327680.0) * 1024)         # 675.4 MB, 1.0033 x algorithmic (q and k in one launch)
 
 
 # ------------------------------------------------------------------------------------- workloads
