@@ -369,6 +369,32 @@ def test_a_narrowing_op_runs_on_the_side_of_its_input(sa, lib):
     assert not sa.sideaware_last_error()
 
 
+def test_a_batch_of_narrowing_segments_is_sided_segment_by_segment(sa, lib):
+    """Several arrays in one launch of a narrowing op: every segment follows its own input (its
+    own arena constants and origin), so in each of them an input granule is handled by one XCD of
+    the half of the device that holds it."""
+    from l2_torch_alloc_amd import ops
+    kid = sa.sideaware_create_kernel(NARROWING_XCD_ID_HEADER)
+    sizes = [12 * MiB, 8 * MiB + 2048, 20 * MiB]              # elements; the middle one ends in a partial tile
+    srcs = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in sizes]
+    outs = [torch.full((n,), -1, dtype=torch.int16, device="cuda") for n in sizes]
+    segments = [(n * 4, [o], [x], None, 0) for n, o, x in zip(sizes, outs, srcs)]
+    for _ in range(3):
+        before = counts(lib)
+        ops.elementwise_batch(kid, segments)
+        torch.cuda.synchronize()
+        assert counts(lib) == (before[0] + 1, before[1])
+    for n, o, x in zip(sizes, outs, srcs):
+        assert int(o.min()) >= 0 and int(o.max()) <= 7
+        whole = n // 2048 * 2048
+        xcd = o[:whole].view(-1, 2048)                         # one row per input granule
+        assert bool((xcd == xcd[:, :1]).all())
+        half = (xcd[:, 0] // 4).cpu().tolist()
+        for g in range(0, len(half), 53):
+            assert half[g] == lib.sideaware_side_of(x.data_ptr() + g * 8192), (n, g)
+    assert not sa.sideaware_last_error()
+
+
 def test_a_widening_op_is_striped_unless_asked_and_then_follows_its_input(sa, lib):
     """short in, int out (every input narrower than the output): striped by default, which is as
     fast for such ops; with the `sided_widening` switch the sided map follows the input, so each
