@@ -225,14 +225,15 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * "one_shot", "cache_bytes" (launch parameters) and "nt_store", "wg_threads", "write_through"
  * (1: stores are written through the XCD's private L2; 0: the compiler's write-back stores)
  * (compiled in: after a change every op is compiled afresh on its next launch); "sided" (1: launches
- * whose first output (first input, for an op whose output is narrower) lies in an arena of known sides use
+ * whose first input (first output, for an op that has no input as wide) lies in an arena of known sides use
  * the sided map, 0: never), "sided_min_bytes" (arrays
  * shorter than this never do), "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
  * -1: by array size), "sided_wrong" (1: sided launches give every XCD the granules of the other half
  * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,
  * every access crossing between the dies) and "sided_widening" (1: an op whose every input is narrower
  * than its output is sided too, following its first input; 0, the default: such ops use the striped map,
- * which is as fast for them).
+ * which is as fast for them) and "sided_agreement" (per cent of its length over which a second input as
+ * wide as the followed one must have the same sides for the launch to be sided; default 70).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -9,8 +9,8 @@
 // *placement guarantee*: every large region starts on a kRegionAlign (2 MiB) boundary, and regions
 // of kCanonicalMinBytes or more start where the backing store says the sides alternate through
 // them in one common pattern (Backing::place_canonical), so that offset o of any two such regions
-// lies on the same side and an elementwise kernel that follows its output's sides finds its input
-// there too.  The pool delivers that, plus the reference's caching behaviour:
+// lies on the same side and an elementwise kernel that follows the sides of one of its arrays finds the
+// others there too.  The pool delivers that, plus the reference's caching behaviour:
 //
 //   large  (size >= threshold): a 2 MiB-aligned region, size rounded up to 2 MiB.  Freed regions
 //          go to an exact-size LIFO reuse cache, as in the reference: the same size comes back at

@@ -96,22 +96,24 @@ struct Tuning {
     long long sided_stripe = -1;     // log2(pairs per stripe of an XCD) of the sided map; -1: by array size
     long long sided_wrong = 0;       // 1: sided launches give every XCD the granules of the *other* half (an A/B switch)
     long long sided_widening = 0;    // 1: ops whose every input is narrower than the output are sided too, following i0 (an A/B switch)
+    long long sided_agreement = 70;  // per cent of an array over which another array of the same width must match its sides
 };
 
 // The knobs themselves: written by sideaware_tune (and once from the environment), read by every
 // launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
 // a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
-constexpr int kTuneKnobs = 14;
+constexpr int kTuneKnobs = 15;
 static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
                                                    "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd",
                                                    "write_through", "sided", "sided_min_bytes", "sided_stripe",
-                                                   "sided_wrong", "sided_widening"};
+                                                   "sided_wrong", "sided_widening", "sided_agreement"};
 static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
                                                  "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
                                                  "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD",
                                                  "SIDEAWARE_WRITE_THROUGH", "SIDEAWARE_SIDED", "SIDEAWARE_SIDED_MIN_BYTES",
-                                                 "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG", "SIDEAWARE_SIDED_WIDENING"};
-static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}, {0}};
+                                                 "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG", "SIDEAWARE_SIDED_WIDENING",
+                                                 "SIDEAWARE_SIDED_AGREEMENT"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}, {0}, {70}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -143,6 +145,7 @@ static Tuning tuning_snapshot() {
     t.sided_stripe = g_tune[11].load(std::memory_order_relaxed);
     t.sided_wrong = g_tune[12].load(std::memory_order_relaxed);
     t.sided_widening = g_tune[13].load(std::memory_order_relaxed);
+    t.sided_agreement = g_tune[14].load(std::memory_order_relaxed);
     return t;
 }
 
@@ -743,16 +746,19 @@ static unsigned int followed_vector_bytes(const CompiledKernel* k) {
 }
 
 // Whether this launch of the sided instantiation `k` may go ahead, and with which arena constants.
-// A sided launch follows one array (the kernel template says which: o0 for an op whose i0 is as wide,
-// i0 for one that narrows or only widens; num_bytes is the length of the widest array): it must lie in
-// an arena whose sides were measured and start on a granule boundary.  Every other array that is as wide and accessed at the same index (outputs;
-// inputs unless gathered through a custom `indexing`) is then on the right half of the device
-// wherever its side pattern matches the followed array's, and on the wrong half wherever it does not
-// (every access crossing between the dies).  Measured with a 256 MiB copy: all matching 6.9 TB/s, none
-// matching 6.3, the striped map 6.7, so the sided map still wins with up to two fifths of the array
-// mismatched.  Such an array must therefore lie in an arena of known sides and match over at least
-// seven tenths of its length (the patterns are piecewise constant between carries into the hash
-// bits: 64 samples see them).  Narrower arrays fall where they fall: half of their traffic crosses.
+// A sided launch follows one array (the kernel template says which: i0 for an op whose first input is
+// at least as wide as its first output, o0 for a fill or an op with a wider second input; num_bytes is
+// the length of the widest array): it must lie in an arena whose sides were measured and start on a
+// granule boundary.  Every other array that is as wide and accessed at the same index is then on the
+// right half of the device wherever its side pattern matches the followed array's, and on the wrong
+// half wherever it does not (every access crossing between the dies).  For stores that costs little
+// (they are posted: a 256 MiB copy whose destination has the opposite pattern of its source still
+// runs at 6.75 TB/s, above the striped map's 6.70), so outputs are not looked at.  For loads it costs
+// a lot (6.26 TB/s when the followed array is the destination and every load crosses), so an input
+// other than the followed array must lie in an arena of known sides and match over at least seven
+// tenths of its length (the patterns are piecewise constant between carries into the hash bits:
+// 64 samples see them), or the launch uses the striped map.  Narrower arrays fall where they fall:
+// half of their traffic crosses.
 static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const void* const out[4], const void* const in[4],
                             size_t num_bytes, const Tuning& t, SideMap* map) {
     SideRegistry& sides = ctx->backing->sides();
@@ -778,16 +784,12 @@ static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const v
             const unsigned int b = side_parity(((uintptr_t)owner - owner_base + off) & hash.address_mask) ^ owner_flip;
             agree += a == b;
         }
-        return agree * 10 >= kSamples * 7;
+        return agree * 100 >= kSamples * (int)t.sided_agreement;
     };
     for (int j = 0; j < 4; j++) {
         if (!in[j] || k->in_size[j] != owner_size) continue;
         if (j > 0 && k->gathered) continue;
         if (!follows(in[j])) return false;
-    }
-    for (int j = 0; j < 4; j++) {
-        if (!out[j] || k->out_size[j] != owner_size) continue;
-        if (!follows(out[j])) return false;
     }
     // An op that only widens (every input narrower than the output: an MXFP8 -> bf16 dequantise)
     // would follow its input, but gains nothing from it: two thirds of its traffic are stores, half of

@@ -125,10 +125,15 @@ def test_which_launches_are_sided(sa, lib):
     assert copy(dst.data_ptr(), src.data_ptr(), 4 * MiB) == (0, 1)           # too short to matter
     assert copy(dst.data_ptr() + 4096, src.data_ptr() + 4096, n - 8192) == (0, 1)      # not on a granule boundary
     assert torch.equal(dst, src)
-    # the source's sides are the opposite of the destination's over the whole array: every load
-    # would cross between the dies, so the striped map is used
-    assert copy(dst.data_ptr(), src.data_ptr() + 2 * MiB, n - 2 * MiB) == (0, 1)
+    # the source's sides are the opposite of the destination's over the whole array: the launch
+    # follows its source (loads stay on their own half, every store crosses: still faster than stripes)
+    assert copy(dst.data_ptr(), src.data_ptr() + 2 * MiB, n - 2 * MiB) == (1, 0)
     assert torch.equal(dst[: n - 2 * MiB], src[2 * MiB:])
+    # ... wherever the destination lies: only the source has to be on a granule boundary in measured memory
+    dst.zero_()
+    assert copy(dst.data_ptr() + 4096 + 16, src.data_ptr(), n - 8192) == (1, 0)
+    assert torch.equal(dst[4096 + 16: 4096 + 16 + n - 8192], src[: n - 8192])
+    assert copy(dst.data_ptr(), src.data_ptr(), n) == (1, 0)
     assert lib.sideaware_tune(b"sided", 0) == 0
     assert copy(dst.data_ptr(), src.data_ptr(), n) == (0, 1)
     assert lib.sideaware_tune(b"sided", 1) == 0
@@ -242,8 +247,9 @@ def test_sided_copy_is_bit_exact_whatever_the_host_believes(sa, lib, nbytes):
 
 def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
     """An op that stores the id of the XCD it runs on: after the stream's dealing offset has been
-    fed back (one launch), every 8 KiB granule of the output was written from the half of the
-    device that sideaware_side_of names for it, and with the wrong-side switch from the other."""
+    fed back (one launch), every 8 KiB granule was handled by the half of the device that
+    sideaware_side_of names for that granule of the source (the array a launch follows), and with the
+    wrong-side switch by the other."""
     stream = torch.cuda.current_stream().cuda_stream
     kid = sa.sideaware_create_kernel(XCD_ID_HEADER)
     n = 64 * MiB
@@ -263,7 +269,7 @@ def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
         step = 97
         checked = 0
         for g in range(0, len(half), step):
-            side = lib.sideaware_side_of(out.data_ptr() + g * 8192)
+            side = lib.sideaware_side_of(src.data_ptr() + g * 8192)
             assert side in (0, 1)
             assert half[g] == side ^ wrong, (g, half[g], side, wrong)
             checked += 1
@@ -318,7 +324,7 @@ def test_the_dealing_offset_survives_other_kernels_on_the_stream(sa, lib):
     n = 32 * MiB
     src = torch.zeros(n // 4, dtype=torch.int32, device="cuda")
     out = torch.full((n // 4,), -1, dtype=torch.int32, device="cuda")
-    sides = torch.tensor([lib.sideaware_side_of(out.data_ptr() + g * 8192) for g in range(0, n // 8192, 61)], device="cuda")
+    sides = torch.tensor([lib.sideaware_side_of(src.data_ptr() + g * 8192) for g in range(0, n // 8192, 61)], device="cuda")
     assert int(sides.min()) >= 0
 
     def launch():

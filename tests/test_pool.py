@@ -490,8 +490,8 @@ def test_large_regions_share_one_side_pattern(ph):
     """With a backing store that knows which half of the device holds which 8 KiB granule (the HIP
     one measures it), regions of 32 MiB and more are placed so that the granule at offset o is on
     side parity(o & bits 13, 21, 28) in every one of them, whatever arena they come from and
-    whatever lies around them: an elementwise kernel that follows its output's sides then finds
-    its input on the same side."""
+    whatever lies around them: an elementwise kernel that follows the sides of one of its arrays then finds
+    the others on the same side."""
     SIDE_BITS = (1 << 13) | (1 << 21) | (1 << 28)
     p = P(ph, capacity=256 * GiB, arena=4 * GiB)
     ph.ph_set_side_rule(p.h, 1)
