@@ -232,8 +232,9 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,
  * every access crossing between the dies) and "sided_widening" (1: an op whose every input is narrower
  * than its output is sided too, following its first input; 0, the default: such ops use the striped map,
- * which is as fast for them) and "sided_agreement" (per cent of its length over which a second input as
- * wide as the followed one must have the same sides for the launch to be sided; default 70).
+ * which is as fast for them) "sided_agreement" (per cent of its length over which a second input as
+ * wide as the followed one must have the same sides for the launch to be sided; default 70) and
+ * "sided_align" (the followed array must start on a multiple of this many bytes; default 16).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -83,7 +83,7 @@ def lib(sa):
         pytest.skip("the device showed no side structure to the start-up probe")
     yield L
     for key, value in ((b"sided", 1), (b"sided_wrong", 0), (b"sided_stripe", -1), (b"sided_min_bytes", 8 * MiB),
-                       (b"sided_widening", 0)):
+                       (b"sided_widening", 0), (b"sided_align", 16), (b"sided_agreement", 70)):
         assert L.sideaware_tune(key, value) == 0
 
 
@@ -123,13 +123,17 @@ def test_which_launches_are_sided(sa, lib):
     assert copy(dst.data_ptr(), src.data_ptr(), n) == (1, 0)                 # two canonical regions: sided
     assert torch.equal(dst, src)
     assert copy(dst.data_ptr(), src.data_ptr(), 4 * MiB) == (0, 1)           # too short to matter
-    assert copy(dst.data_ptr() + 4096, src.data_ptr() + 4096, n - 8192) == (0, 1)      # not on a granule boundary
+    assert copy(dst.data_ptr() + 4096, src.data_ptr() + 4096, n - 8192) == (1, 0)      # not on a granule boundary: still sided
+    assert copy(dst.data_ptr() + 1024 + 16, src.data_ptr() + 1024 + 16, n - 8192) == (1, 0)
+    assert lib.sideaware_tune(b"sided_align", 8192) == 0                               # unless an alignment is demanded
+    assert copy(dst.data_ptr() + 4096, src.data_ptr() + 4096, n - 8192) == (0, 1)
+    assert lib.sideaware_tune(b"sided_align", 16) == 0
     assert torch.equal(dst, src)
     # the source's sides are the opposite of the destination's over the whole array: the launch
     # follows its source (loads stay on their own half, every store crosses: still faster than stripes)
     assert copy(dst.data_ptr(), src.data_ptr() + 2 * MiB, n - 2 * MiB) == (1, 0)
     assert torch.equal(dst[: n - 2 * MiB], src[2 * MiB:])
-    # ... wherever the destination lies: only the source has to be on a granule boundary in measured memory
+    # ... wherever the destination lies: only the source has to be in measured memory
     dst.zero_()
     assert copy(dst.data_ptr() + 4096 + 16, src.data_ptr(), n - 8192) == (1, 0)
     assert torch.equal(dst[4096 + 16: 4096 + 16 + n - 8192], src[: n - 8192])
@@ -190,7 +194,7 @@ __device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *o
     torch.cuda.synchronize()
     assert counts(lib) == (before[0] + 1, before[1]) and int(hits[0]) == 2
     # an op whose output is narrower than its input follows the input: the input must be in measured
-    # memory and start on a granule boundary, the output may be anywhere
+    # memory, the output may be anywhere
     narrow = sa.sideaware_create_kernel(NARROWING_XCD_ID_HEADER)
     w = torch.zeros(16 * MiB, device="cuda")
     h = torch.empty(16 * MiB + 8, dtype=torch.int16, device="cuda")
@@ -201,7 +205,7 @@ __device__ __forceinline__ void vector_op(size_type vec_idx, int vec_size, o0 *o
     before = counts(lib)
     lib.sideaware_one_to_one(narrow, w.numel() * 4 - 8192, h.data_ptr(), w.data_ptr() + 4096, 0, stream)
     torch.cuda.synchronize()
-    assert counts(lib) == (before[0], before[1] + 1)
+    assert counts(lib) == (before[0] + 1, before[1])
 
 
 def agreeing_offset(lib, base, nbytes, first):
@@ -246,9 +250,9 @@ def test_sided_copy_is_bit_exact_whatever_the_host_believes(sa, lib, nbytes):
 
 
 def test_sided_copies_at_random_offsets_are_bit_exact(sa, lib):
-    """Seeded random lengths, source offsets (granule-aligned, so the launch is sided) and
-    destination offsets (any multiple of 16 bytes: aligned and split-line stores, matching and
-    opposite side patterns): every byte arrives, none beside the destination changes."""
+    """Seeded random lengths, source offsets (on and off granule boundaries) and destination
+    offsets (any multiple of 16 bytes: aligned and split-line stores, matching and opposite side
+    patterns): every launch is sided, every byte arrives, none beside the destination changes."""
     import random
     stream = torch.cuda.current_stream().cuda_stream
     rng = random.Random(20)
@@ -257,7 +261,7 @@ def test_sided_copies_at_random_offsets_are_bit_exact(sa, lib):
     sided = 0
     for case in range(24):
         n = rng.randrange(8 * MiB, 96 * MiB) // 16 * 16
-        s_off = rng.randrange(0, 2 * MiB // 8192) * 8192
+        s_off = rng.randrange(0, 2 * MiB // 8192) * 8192 + rng.choice([0, 0, 16, 64, 1024, 4096, 4096 + 48])
         d_off = rng.choice([0, 16, 64, 4096, 8192, 2 * MiB]) + rng.randrange(0, 4096 // 16) * 16 * rng.choice([0, 1])
         d_off = max(d_off, 64)                     # room for guard bytes in front
         big_dst.fill_(0xA5)
