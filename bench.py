@@ -298,6 +298,42 @@ def bench_one_direction(nbytes=GiB, sets=4, steps=12, rounds=3):
     return out
 
 
+def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
+    """Producer -> consumer chains: three buffers, every launch copies the one the launch before it
+    wrote into the next, so each launch reads what was just written (from the Infinity Cache while
+    three buffers fit it, partly from HBM at 256 MiB).  Sided and XCD-striped in turn (medians)."""
+    import torch
+    lib, stream = _abi()
+    out = {}
+    for nbytes in sizes:
+        bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(3)]
+        first = bufs[0].clone()
+        counter = [0]
+
+        def launch():
+            i = counter[0] % 3
+            counter[0] += 1
+            lib.sideaware_memcpy(bufs[(i + 1) % 3].data_ptr(), bufs[i].data_ptr(), nbytes, 0, stream)
+
+        times = {1: [], 0: []}
+        n_steps = max(30, steps * (16 * MiB) // nbytes)
+        try:
+            for _ in range(rounds):
+                for sided in (1, 0):
+                    lib.sideaware_tune(b"sided", sided)
+                    times[sided].append(time_region(launch, n_steps, 9))
+        finally:
+            lib.sideaware_tune(b"sided", 1)
+        ok = all(bool(torch.equal(b, first)) for b in bufs)
+        entry = {"bytes": nbytes, "bit_exact": ok}
+        for sided, name in ((1, "sided"), (0, "xcd_striped")):
+            sec = statistics.median(times[sided])
+            entry[name] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes, sec)}
+        out["%dMiB" % (nbytes // MiB)] = entry
+        del bufs
+    return out
+
+
 def bench_vendor_copies(nbytes, pairs, steps):
     """The same cycling copy done by the platform's own copy paths, for scale: PyTorch's copy_
     kernel and the runtime's device-to-device hipMemcpyAsync, on the same kind of buffers."""
@@ -949,6 +985,8 @@ def main():
         also["copy_sweep"] = sweep
         also["copy_256MiB_ownership_map_ab"] = bench_side_ab()
         log("ownership map A/B:", also["copy_256MiB_ownership_map_ab"])
+        also["chain_each_launch_reads_what_the_last_wrote"] = bench_chains()
+        log("chains:", also["chain_each_launch_reads_what_the_last_wrote"])
         also["one_direction_1GiB"] = bench_one_direction()
         log("one direction only:", also["one_direction_1GiB"])
         also["copy_4MiB_replayed_from_a_hip_graph"] = bench_small_copy_in_graph()
