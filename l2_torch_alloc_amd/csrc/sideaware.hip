@@ -725,10 +725,23 @@ static long long slots_wanted_for(const DeviceContext* ctx, const CompiledKernel
 // sided (see sa_sided_possible in the kernel template), and one of the two arrays a sided launch may
 // follow lies in an arena whose sides were measured (and starts on a multiple of the `sided_align` knob).
 static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const void* out0, const void* in0,
-                            size_t num_bytes, const Tuning& t) {
+                            size_t num_bytes, const Tuning& t, sideaware_stream_t stream) {
     if (!t.sided || num_bytes < (unsigned long long)t.sided_min_bytes) return false;
     if (entry->sided_possible.load(std::memory_order_relaxed) == 0) return false;
     if (ctx->num_xcds < 2 || (ctx->num_xcds & (ctx->num_xcds - 1))) return false;
+    // A launch that is being captured into a graph will run later, on whatever queue the graph is
+    // replayed through, and the workgroups of a replayed node are dealt to the XCDs from another
+    // offset than those of a launch made directly on any stream (measured: 5 or 6 where the capture
+    // stream and the replay stream report 0 and 7).  A sided plan made with the wrong offset sends most
+    // accesses across the dies (a replayed 256 MiB copy: 0.56 of the HBM peak, 0.83 striped), and the
+    // offset is frozen into the node's arguments, so captured launches use the map that does not
+    // depend on it.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (capturing != hipStreamCaptureStatusNone) return false;
     const uintptr_t kGranuleMask = (uintptr_t)(t.sided_align > 16 ? t.sided_align : 16) - 1;
     SideRegistry& sides = ctx->backing->sides();
     uintptr_t base = 0;
@@ -946,7 +959,7 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     if (!entry) return;
     SideMap side;
     const CompiledKernel* k = nullptr;
-    if (sided_candidate(ctx, entry, out0, in0, num_bytes, t)) {
+    if (sided_candidate(ctx, entry, out0, in0, num_bytes, t, stream)) {
         k = get_kernel(ctx, kernel_id, variant | kVariantSided);
         const void* const outs[4] = {out0, out1, out2, out3};
         const void* const ins[4] = {in0, in1, in2, in3};
@@ -1056,7 +1069,7 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
         SideMap sides[kMaxSegments];
         bool all_sided = true;
         for (int i = 0; i < count && all_sided; i++) {
-            all_sided = sided_candidate(ctx, entry, group[i]->out[0], group[i]->in[0], group[i]->num_bytes, t);
+            all_sided = sided_candidate(ctx, entry, group[i]->out[0], group[i]->in[0], group[i]->num_bytes, t, stream);
         }
         const CompiledKernel* k = nullptr;
         if (all_sided) {

@@ -310,16 +310,20 @@ def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
     assert 0 <= lib.sideaware_stream_dealing(stream) <= 7
 
 
-def test_sided_launches_replay_from_a_hip_graph(sa, lib):
-    """A sided launch under stream capture: the dealing offset the host believed at capture time
-    is frozen into the graph's kernel arguments; whatever the stream does on later replays, every
-    replay is bit-exact (the map is a bijection for any belief), also with eager work between them."""
+def test_launches_captured_into_a_hip_graph_use_the_striped_map(sa, lib):
+    """The workgroups of a replayed graph node are dealt to the XCDs from another offset than
+    those of a direct launch, and a captured launch's plan is frozen, so a launch under stream
+    capture is planned with the map that does not depend on the offset (a sided plan with the wrong
+    offset would run at two thirds of the striped map's speed).  Replays are bit-exact, also with
+    eager, sided work of the program's own between them."""
     n = 64 * MiB
     src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
     mid = torch.zeros_like(src)
     dst = torch.zeros_like(src)
-    torch.ops.sideaware.memcpy(mid, src)            # compiles the instantiation outside the capture
+    before = counts(lib)
+    torch.ops.sideaware.memcpy(mid, src)            # compiles outside the capture; sided
     torch.cuda.synchronize()
+    assert counts(lib) == (before[0] + 1, before[1])
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -329,12 +333,14 @@ def test_sided_launches_replay_from_a_hip_graph(sa, lib):
             torch.ops.sideaware.memcpy(mid, src)
             torch.ops.sideaware.memcpy(dst, mid)
     torch.cuda.current_stream().wait_stream(side)
-    assert counts(lib)[0] == before[0] + 2, "the captured launches were not sided"
+    assert counts(lib) == (before[0], before[1] + 2), "the captured launches were planned sided"
     other = torch.zeros(16 * MiB, dtype=torch.uint8, device="cuda")
     for trial in range(4):
         src.random_(0, 256)
         dst.zero_()
+        before = counts(lib)
         torch.ops.sideaware.memcpy(other, src[: 16 * MiB])      # eager work of the program's own between replays
+        assert counts(lib) == (before[0] + 1, before[1])
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
