@@ -197,6 +197,10 @@ unsigned long long sideaware_side_address_mask(void);
 int sideaware_side_of(const void* ptr);
 int sideaware_stream_dealing(sideaware_stream_t stream);
 void sideaware_launch_counts(unsigned long long* sided, unsigned long long* striped);
+/* Overrides what the stream's last sided launch reported (no counterpart in the reference): for a
+ * host that knows which XCD workgroup 0 of its next launch will run on, and for tests.  A stream
+ * whose reported offset keeps changing from launch to launch gets the striped map until it settles. */
+void sideaware_set_stream_dealing(sideaware_stream_t stream, int dealing);
 /* Text of the most recent failure on any thread ("" if none).  The pointer is the calling thread's
  * own copy, valid until that thread calls again. */
 const char* sideaware_last_error(void);

@@ -121,7 +121,15 @@ public:
 
     // Where workgroup 0 of a sided launch on `stream` reports its XCD (pinned host memory the
     // device can write), and the dealing offset last reported there (0 before the first report).
-    unsigned int* feedback_slot(void* stream, unsigned int* dealing);
+    // `account` says the caller is planning a launch with the answer (a query passes false).
+    unsigned int* feedback_slot(void* stream, unsigned int* dealing, bool account = true);
+    // False while the offsets reported for `stream` keep changing from one launch to the next (a
+    // stream that is moved between hardware queues): a sided plan would then be made with the wrong
+    // offset most of the time, which is worse than no plan.  Every call while unsteady counts towards
+    // trying again.
+    bool stream_is_steady(void* stream);
+    // Writes `dealing` where the stream's kernels report (as if a launch had just reported it).
+    void report_dealing(void* stream, unsigned int dealing);
 
     // Times loads from every XCD at `count` sample granules of [region, region + bytes) on
     // `stream` and writes, for each, the side that is clearly nearer (0 or 1), or -1, to the device
@@ -171,6 +179,14 @@ private:
     unsigned int* static_scratch_ = nullptr;        // this device's address of the static work array
     std::unordered_map<void*, int> slot_of_stream_;
     static constexpr int kFeedbackSlots = 64;
+    struct SlotState {
+        unsigned int believed = 0;
+        bool has = false;
+        int flaps = 0;             // +4 for every change of the reported offset, -1 for every launch without (0..32)
+    };
+    SlotState slot_state_[kFeedbackSlots];
+    static constexpr int kUnsteadyFlaps = 12;
+    int slot_of_locked(void* stream);
     static constexpr int kMaxProbe = 512;
 };
 

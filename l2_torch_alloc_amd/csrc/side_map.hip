@@ -531,23 +531,51 @@ int SideRegistry::side_of(const void* addr) {
     return (int)(side_parity(((uintptr_t)addr - base) & h.address_mask) ^ flip);
 }
 
-unsigned int* SideRegistry::feedback_slot(void* stream, unsigned int* dealing) {
+int SideRegistry::slot_of_locked(void* stream) {
+    auto it = slot_of_stream_.find(stream);
+    if (it != slot_of_stream_.end()) return it->second;
+    // more streams than slots: the late ones share the last slot (and each other's reports)
+    const int slot = (int)slot_of_stream_.size() < kFeedbackSlots ? (int)slot_of_stream_.size() : kFeedbackSlots - 1;
+    slot_of_stream_.emplace(stream, slot);
+    return slot;
+}
+
+unsigned int* SideRegistry::feedback_slot(void* stream, unsigned int* dealing, bool account) {
     std::lock_guard<std::mutex> g(mu_);
     *dealing = 0;
     if (!ensure_feedback_locked()) return nullptr;
-    int slot;
-    auto it = slot_of_stream_.find(stream);
-    if (it != slot_of_stream_.end()) {
-        slot = it->second;
-    } else {
-        // more streams than slots: the late ones share the last slot (and each other's reports)
-        slot = (int)slot_of_stream_.size() < kFeedbackSlots ? (int)slot_of_stream_.size() : kFeedbackSlots - 1;
-        slot_of_stream_.emplace(stream, slot);
-    }
+    const int slot = slot_of_locked(stream);
     volatile unsigned int* word = feedback_ + (size_t)slot * 16;
     const unsigned int v = *word;
-    if (v & 0x80000000u) *dealing = v & 0xfu;
+    if (v & 0x80000000u) {
+        SlotState& st = slot_state_[slot];
+        const unsigned int k = v & 0xfu;
+        *dealing = k;
+        if (account) {
+            if (st.has && k != st.believed) st.flaps = st.flaps + 4 > 32 ? 32 : st.flaps + 4;
+            else if (st.flaps > 0) st.flaps--;
+            st.believed = k;
+            st.has = true;
+        }
+    }
     return (unsigned int*)word;
+}
+
+bool SideRegistry::stream_is_steady(void* stream) {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = slot_of_stream_.find(stream);
+    if (it == slot_of_stream_.end()) return true;
+    SlotState& st = slot_state_[it->second];
+    if (st.flaps < kUnsteadyFlaps) return true;
+    st.flaps--;                                      // this launch goes striped; a few of those and sided is tried again
+    return false;
+}
+
+void SideRegistry::report_dealing(void* stream, unsigned int dealing) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (!ensure_feedback_locked()) return;
+    volatile unsigned int* word = feedback_ + (size_t)slot_of_locked(stream) * 16;
+    *word = 0x80000000u | (dealing & 0xfu);
 }
 
 }  // namespace sideaware

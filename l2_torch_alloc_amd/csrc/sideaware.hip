@@ -742,6 +742,7 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
         return false;
     }
     if (capturing != hipStreamCaptureStatusNone) return false;
+    if (!ctx->backing->sides().stream_is_steady(stream)) return false;
     const uintptr_t kGranuleMask = (uintptr_t)(t.sided_align > 16 ? t.sided_align : 16) - 1;
     SideRegistry& sides = ctx->backing->sides();
     uintptr_t base = 0;
@@ -1255,7 +1256,7 @@ int sideaware_stream_dealing(sideaware_stream_t stream) {
     DeviceContext* c = get_context();
     if (!c) return -1;
     unsigned int dealing = 0;
-    return c->backing->sides().feedback_slot(stream, &dealing) ? (int)dealing : -1;
+    return c->backing->sides().feedback_slot(stream, &dealing, /*account=*/false) ? (int)dealing : -1;
 }
 
 static int probe_sides_common(const char* what, const void* region, size_t num_bytes, unsigned long long seed, int count,
@@ -1283,6 +1284,12 @@ int sideaware_probe_sides(const void* region, size_t num_bytes, unsigned long lo
 int sideaware_probe_sides_noalloc(const void* region, size_t num_bytes, unsigned long long seed, int count, int* sides,
                                   int device, sideaware_stream_t stream) {
     return probe_sides_common("probe_sides_noalloc", region, num_bytes, seed, count, sides, device, stream, /*allocate=*/false);
+}
+
+void sideaware_set_stream_dealing(sideaware_stream_t stream, int dealing) {
+    DeviceContext* c = get_context();
+    if (!c || dealing < 0) return;
+    c->backing->sides().report_dealing(stream, (unsigned int)dealing % (unsigned int)(c->num_xcds > 0 ? c->num_xcds : 1));
 }
 
 int sideaware_register_region(void* region, size_t num_bytes, int device) {

@@ -78,6 +78,7 @@ _SIGNATURES = {
     "sideaware_side_address_mask": (ctypes.c_ulonglong, []),
     "sideaware_side_of": (_ci, [_vp]),
     "sideaware_stream_dealing": (_ci, [_vp]),
+    "sideaware_set_stream_dealing": (None, [_vp, _ci]),
     "sideaware_launch_counts": (None, [ctypes.POINTER(ctypes.c_ulonglong), ctypes.POINTER(ctypes.c_ulonglong)]),
     "sideaware_last_error": (ctypes.c_char_p, []),
     "sideaware_clear_error": (None, []),

@@ -383,6 +383,40 @@ def test_the_dealing_offset_survives_other_kernels_on_the_stream(sa, lib):
         assert believed == reported and wrong == 0, (trial, believed, reported, wrong)
 
 
+def test_a_stream_whose_offset_keeps_changing_goes_striped_until_it_settles(sa, lib):
+    """The host plans a sided launch with the offset the stream's last sided launch reported.  A
+    stream that reports another offset at every launch (forced here by overwriting the report, as a
+    stream moved between hardware queues would) makes every plan wrong, so after a few changes its
+    launches use the striped map, and go back to the sided one once the reports agree again.
+    Results are exact throughout."""
+    side = torch.cuda.Stream()
+    stream = side.cuda_stream
+    n = 32 * MiB
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros_like(src)
+    torch.cuda.synchronize()
+
+    def launch():
+        before = counts(lib)
+        lib.sideaware_memcpy(dst.data_ptr(), src.data_ptr(), n, 0, stream)
+        side.synchronize()
+        after = counts(lib)
+        return after[0] - before[0]
+
+    assert [launch() for _ in range(4)] == [1, 1, 1, 1]
+    true_offset = lib.sideaware_stream_dealing(stream)
+    used = []
+    for i in range(12):
+        lib.sideaware_set_stream_dealing(stream, (true_offset + 1 + i % 3) % 8)     # never what the launch will report
+        used.append(launch())
+    assert used[:3] == [1, 1, 1] and 0 in used[3:], used
+    assert sum(used[4:]) <= 3, used                      # mostly striped once the changes were noticed
+    settled = [launch() for _ in range(24)]
+    assert settled[-4:] == [1, 1, 1, 1], settled
+    assert lib.sideaware_stream_dealing(stream) == true_offset
+    assert torch.equal(dst, src)
+
+
 def test_a_narrowing_op_runs_on_the_side_of_its_input(sa, lib):
     """float in, short out: the sided map follows the input (the wider array, two thirds of the
     traffic).  Every 8 KiB granule of the input is read, and its 4 KiB of output written, by an XCD
