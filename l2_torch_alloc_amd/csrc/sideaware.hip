@@ -794,10 +794,13 @@ static bool sided_launch_ok(DeviceContext* ctx, const CompiledKernel* k, const v
         uintptr_t base = 0;
         unsigned int flip = 0;
         if (!sides.arena_of(p, &base, &flip)) return false;
+        // samples spread over the array and over the low address bits (an array that is another one
+        // moved by less than a page differs from it only where the move carries into a hash bit)
         constexpr int kSamples = 64;
+        const uint64_t granules = owner_bytes >> kSideGranuleLog2;
         int agree = 0;
         for (int i = 0; i < kSamples; i++) {
-            const uint64_t off = (uint64_t)(owner_bytes / kSamples) * (unsigned)i;
+            const uint64_t off = granules ? (((uint64_t)(unsigned)i * 0x9e3779b97f4a7c15ull >> 20) % granules) << kSideGranuleLog2 : 0;
             const unsigned int a = side_parity(((uintptr_t)p - base + off) & hash.address_mask) ^ flip;
             const unsigned int b = side_parity(((uintptr_t)owner - owner_base + off) & hash.address_mask) ^ owner_flip;
             agree += a == b;
