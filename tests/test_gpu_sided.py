@@ -275,14 +275,15 @@ def test_sided_copies_at_random_offsets_are_bit_exact(sa, lib):
     assert not sa.sideaware_last_error()
 
 
-def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
+@pytest.mark.parametrize("n", [16 * MiB, 64 * MiB, 256 * MiB, 1024 * MiB])
+def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib, n):
     """An op that stores the id of the XCD it runs on: after the stream's dealing offset has been
     fed back (one launch), every 8 KiB granule was handled by the half of the device that
     sideaware_side_of names for that granule of the source (the array a launch follows), and with the
-    wrong-side switch by the other."""
+    wrong-side switch by the other: what the queries report predicts where the work runs, in every
+    size class of the launch planner (16 MiB, 64 MiB, 256 MiB, 1 GiB)."""
     stream = torch.cuda.current_stream().cuda_stream
     kid = sa.sideaware_create_kernel(XCD_ID_HEADER)
-    n = 64 * MiB
     src = torch.zeros(n // 4, dtype=torch.int32, device="cuda")
     out = torch.full((n // 4,), -1, dtype=torch.int32, device="cuda")
     for wrong in (0, 1):
@@ -296,14 +297,14 @@ def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib):
         assert bool((xcd == xcd[:, :1]).all()), "a granule was written from more than one XCD"
         assert int(xcd.min()) >= 0 and int(xcd.max()) <= 7
         half = (xcd[:, 0] // 4).cpu().tolist()
-        step = 97
+        step = 97 if n <= 64 * MiB else 997
         checked = 0
         for g in range(0, len(half), step):
             side = lib.sideaware_side_of(src.data_ptr() + g * 8192)
             assert side in (0, 1)
             assert half[g] == side ^ wrong, (g, half[g], side, wrong)
             checked += 1
-        assert checked > 50
+        assert checked > 20
         # and the XCDs of a side share the work evenly
         per_xcd = torch.bincount(xcd[:, 0].flatten().cpu(), minlength=8).tolist()
         assert max(per_xcd) - min(per_xcd) <= len(half) // 64, per_xcd
