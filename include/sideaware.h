@@ -157,7 +157,9 @@ int sideaware_xcd_dealing_verified(void);
  * granule at ptr, or -1 for memory outside the pool's arenas or an arena that did not fit the mask.
  * sideaware_stream_dealing: the XCD that workgroup 0 of the last finished sided launch on `stream`
  * ran on (0 before any): sided launches plan with it.  sideaware_launch_counts: launches so far
- * that used the sided map, and launches that used the XCD-striped one. */
+ * that used the sided map, and launches that used the XCD-striped one.  Launches made while their
+ * stream is being captured into a graph always use the striped one (the offset a replayed node sees
+ * is not the one a direct launch sees, and a captured plan cannot follow it). */
 /* Measures which side `count` sample granules of the device memory [region, region + num_bytes)
  * lie on, for memory the pool did not hand out (for the pool's own, sideaware_side_of answers
  * from what was measured when the arena was acquired).  Sample i is the 8 KiB granule number
@@ -234,9 +236,9 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * shorter than this never do), "sided_stripe" (log2 of the pairs of granules an XCD takes in a row;
  * -1: by array size), "sided_wrong" (1: sided launches give every XCD the granules of the other half
  * of the device, the counterpart of the reference's FORCE_WRONG_SIDE, sideaware.cu:70-75: same results,
- * every access crossing between the dies) and "sided_widening" (1: an op whose every input is narrower
+ * every access crossing between the dies), "sided_widening" (1: an op whose every input is narrower
  * than its output is sided too, following its first input; 0, the default: such ops use the striped map,
- * which is as fast for them) "sided_agreement" (per cent of its length over which a second input as
+ * which is as fast for them), "sided_agreement" (per cent of its length over which a second input as
  * wide as the followed one must have the same sides for the launch to be sided; default 70) and
  * "sided_align" (the followed array must start on a multiple of this many bytes; default 16).
  * Returns 0 if the key is known and the value acceptable. */
