@@ -15,8 +15,10 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <map>
 #include <mutex>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 #include "launch_plan.h"
@@ -131,6 +133,19 @@ public:
     // Writes `dealing` where the stream's kernels report (as if a launch had just reported it).
     void report_dealing(void* stream, unsigned int dealing);
 
+    // For a launch on a stream that is being captured into a graph.  The offset from which a
+    // replayed node's workgroups are dealt to the XCDs belongs to the queue the graph is replayed
+    // through, so it cannot be frozen into the node: the node's kernel reads it from a device word
+    // instead, which a one-wave kernel captured ahead of it on the same stream writes at every
+    // replay (launch_plan.h: SideMap::dealing_from_memory).  Returns that word for the capture
+    // `stream` is part of, one word per capture and stream, after capturing the one-wave kernel
+    // if this is the first call for the pair; nullptr when the stream is not being captured, or no
+    // word is left (a process gets kCaptureWords of them and they are never reused: two graphs
+    // sharing a word could write it while the other reads).  *capturing says which.
+    unsigned int* capture_word(void* stream, bool* capturing);
+    void init_capture_words();
+    static constexpr int kCaptureWords = 4096;
+
     // Times loads from every XCD at `count` sample granules of [region, region + bytes) on
     // `stream` and writes, for each, the side that is clearly nearer (0 or 1), or -1, to the device
     // array `sides`.  With allocate == false nothing is allocated: the work space is a static
@@ -185,6 +200,9 @@ private:
         int flaps = 0;             // +4 for every change of the reported offset, -1 for every launch without (0..32)
     };
     SlotState slot_state_[kFeedbackSlots];
+    unsigned int* capture_words_ = nullptr;         // this device's address of the static word array
+    int capture_words_used_ = 0;
+    std::map<std::pair<unsigned long long, void*>, int> capture_word_of_;   // (capture id, stream) -> word
     static constexpr int kUnsteadyFlaps = 12;
     int slot_of_locked(void* stream);
     static constexpr int kMaxProbe = 512;

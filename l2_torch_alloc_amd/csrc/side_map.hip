@@ -180,6 +180,54 @@ void SideRegistry::init_static_scratch() {
     static_scratch_ = (unsigned int*)ptr;            // this device's copy of the array
 }
 
+// The words captured launches read their dealing offset from, and the kernel that writes one: a
+// single wave, captured ahead of the launches that read the word, on the same stream.
+static __device__ __align__(256) unsigned int capture_words[SideRegistry::kCaptureWords];
+
+__global__ __launch_bounds__(64) void sa_scout(unsigned int* word) {
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    if (threadIdx.x == 0) *word = 0x80000000u | (xcc & 0xfu);
+}
+
+void SideRegistry::init_capture_words() {
+    std::lock_guard<std::mutex> g(mu_);
+    if (capture_words_) return;
+    DeviceGuard dev(device_);
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(capture_words)) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    capture_words_ = (unsigned int*)ptr;
+}
+
+unsigned int* SideRegistry::capture_word(void* stream, bool* capturing) {
+    *capturing = false;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    if (hipStreamGetCaptureInfo((hipStream_t)stream, &status, &id) != hipSuccess) {
+        (void)hipGetLastError();
+        *capturing = true;                           // cannot tell: treat as captured, without a word
+        return nullptr;
+    }
+    if (status == hipStreamCaptureStatusNone) return nullptr;
+    *capturing = true;
+    if (status != hipStreamCaptureStatusActive) return nullptr;
+    std::lock_guard<std::mutex> g(mu_);
+    if (!capture_words_) return nullptr;
+    const auto key = std::make_pair(id, stream);
+    auto it = capture_word_of_.find(key);
+    if (it != capture_word_of_.end()) return capture_words_ + it->second;
+    if (capture_words_used_ >= kCaptureWords) return nullptr;
+    unsigned int* word = capture_words_ + capture_words_used_;
+    DeviceGuard dev(device_);
+    hipLaunchKernelGGL(sa_scout, dim3(1), dim3(64), 0, (hipStream_t)stream, word);      // captured, like the launch that follows
+    if (hipGetLastError() != hipSuccess) return nullptr;
+    capture_word_of_.emplace(key, capture_words_used_++);
+    return word;
+}
+
 // The pinned words the sided kernels report their XCD to.  Allocated when the device is set up, so
 // that a first sided launch may happen under stream capture (which allows no allocation).
 bool SideRegistry::ensure_feedback_locked() {

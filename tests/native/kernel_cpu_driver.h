@@ -22,6 +22,10 @@
 #include "../../l2_torch_alloc_amd/csrc/launch_plan.h"
 
 static unsigned g_stripe_log2 = 14, g_slot_run = 1, g_segments = 1;
+// The word a launch planned with `dealing_from_memory` reads its dealing offset from (the driver
+// sets it per case, to a value the plan does not know).
+static unsigned int g_dealing_word = 0;
+static bool g_dealing_from_memory = false;
 
 // The plan for one array: the striped one, or, in an instantiation built with SA_SIDED, the sided
 // one with an origin, arena constant and dealing offset derived from the case (any values must
@@ -33,6 +37,7 @@ static sideaware::LaunchPlan make_plan(unsigned long long base, long long nv, un
         side.pair_mask = SA_SIDE_PAIR_MASK;
         side.flip = (unsigned)(nv & 1);
         side.dealing = (unsigned)((grid + nv + g_stripe_log2) % SA_NUM_XCD);
+        side.dealing_from_memory = g_dealing_from_memory;
         return sideaware::plan_launch_sided(base, nv, sideaware_kernel_meta[0], SA_NUM_XCD, g_stripe_log2 % 9,
                                             g_slot_run, grid / SA_NUM_XCD, side, (unsigned)sa_followed_vector_bytes);
     }
@@ -82,7 +87,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
                 blockIdx = {b, 0, 0};
                 threadIdx = {t, 0, 0};
                 const unsigned* e = batch.blocks_end;
-                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments, nullptr);
+                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments,
+                                               g_dealing_from_memory ? &g_dealing_word : nullptr);
             }
         }
         return;
@@ -96,7 +102,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
             KERNEL_NAME(nv, (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
-                        p.r_word, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem, nullptr);
+                        p.r_word, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem,
+                        g_dealing_from_memory ? &g_dealing_word : nullptr);
         }
     }
 }
@@ -241,6 +248,9 @@ int main() {
         if (std::sscanf(line, "%u %lld %zu %u %u %u", &grid, &nv, &off, &g_stripe_log2, &g_slot_run, &g_segments) < 5) continue;
         if (g_segments < 1 || g_segments > SA_MAX_SEGMENTS) g_segments = 1;
         cases++;
+        // every third case of a sided instantiation takes its dealing offset from memory
+        g_dealing_from_memory = sa_sided && (cases % 3 == 0);
+        g_dealing_word = 0x80000000u | (unsigned)((cases * 5 + nv) % SA_NUM_XCD);
         int bad = run_case(grid, nv, off);
         if (bad) {
             failed++;

@@ -311,20 +311,24 @@ def test_every_workgroup_runs_on_the_side_of_its_bytes(sa, lib, n):
     assert 0 <= lib.sideaware_stream_dealing(stream) <= 7
 
 
-def test_launches_captured_into_a_hip_graph_use_the_striped_map(sa, lib):
+def test_sided_launches_replay_from_a_hip_graph(sa, lib):
     """The workgroups of a replayed graph node are dealt to the XCDs from another offset than
-    those of a direct launch, and a captured launch's plan is frozen, so a launch under stream
-    capture is planned with the map that does not depend on the offset (a sided plan with the wrong
-    offset would run at two thirds of the striped map's speed).  Replays are bit-exact, also with
-    eager, sided work of the program's own between them."""
+    those of a direct launch, and a captured launch's plan is frozen.  So a sided launch under
+    stream capture is preceded (once per capture and stream) by a one-wave kernel that writes the
+    XCD it runs on to a device word, and the launch's own kernel reads its dealing offset from
+    that word at every replay.  Replays are bit-exact on the capture stream, on the default stream
+    and on a third one, also with eager, sided work of the program's own between them, and the XCDs
+    of a replayed launch sit on the side of the bytes they handle."""
     n = 64 * MiB
     src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
     mid = torch.zeros_like(src)
     dst = torch.zeros_like(src)
-    before = counts(lib)
-    torch.ops.sideaware.memcpy(mid, src)            # compiles outside the capture; sided
+    kid = sa.sideaware_create_kernel(XCD_ID_HEADER)
+    zeros = torch.zeros(n // 4, dtype=torch.int32, device="cuda")
+    where = torch.full((n // 4,), -1, dtype=torch.int32, device="cuda")
+    torch.ops.sideaware.memcpy(mid, src)            # compiles outside the capture
+    lib.sideaware_one_to_one(kid, n, where.data_ptr(), zeros.data_ptr(), 0, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert counts(lib) == (before[0] + 1, before[1])
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -333,20 +337,27 @@ def test_launches_captured_into_a_hip_graph_use_the_striped_map(sa, lib):
         with torch.cuda.graph(graph, stream=side):
             torch.ops.sideaware.memcpy(mid, src)
             torch.ops.sideaware.memcpy(dst, mid)
+            lib.sideaware_one_to_one(kid, n, where.data_ptr(), zeros.data_ptr(), 0, side.cuda_stream)
     torch.cuda.current_stream().wait_stream(side)
-    assert counts(lib) == (before[0], before[1] + 2), "the captured launches were planned sided"
+    assert counts(lib) == (before[0] + 3, before[1]), "the captured launches were not sided"
+    sides = torch.tensor([lib.sideaware_side_of(zeros.data_ptr() + g * 8192) for g in range(0, n // 8192, 61)], device="cuda")
     other = torch.zeros(16 * MiB, dtype=torch.uint8, device="cuda")
-    for trial in range(4):
+    third = torch.cuda.Stream()
+    for trial, replay_on in enumerate([torch.cuda.current_stream(), side, third, torch.cuda.current_stream()]):
         src.random_(0, 256)
         dst.zero_()
-        before = counts(lib)
+        where.fill_(-1)
         torch.ops.sideaware.memcpy(other, src[: 16 * MiB])      # eager work of the program's own between replays
-        assert counts(lib) == (before[0] + 1, before[1])
         torch.cuda.synchronize()
-        graph.replay()
+        with torch.cuda.stream(replay_on):
+            graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(dst, src), trial
         assert torch.equal(other, src[: 16 * MiB]), trial
+        xcd = where.view(-1, 2048)
+        assert bool((xcd == xcd[:, :1]).all()) and int(xcd.min()) >= 0 and int(xcd.max()) <= 7, trial
+        wrong = int(((xcd[::61, 0] // 4) != sides).sum())
+        assert wrong == 0, (trial, wrong)
     assert not sa.sideaware_last_error()
 
 
