@@ -157,9 +157,11 @@ int sideaware_xcd_dealing_verified(void);
  * granule at ptr, or -1 for memory outside the pool's arenas or an arena that did not fit the mask.
  * sideaware_stream_dealing: the XCD that workgroup 0 of the last finished sided launch on `stream`
  * ran on (0 before any): sided launches plan with it.  sideaware_launch_counts: launches so far
- * that used the sided map, and launches that used the XCD-striped one.  Launches made while their
- * stream is being captured into a graph always use the striped one (the offset a replayed node sees
- * is not the one a direct launch sees, and a captured plan cannot follow it). */
+ * that used the sided map, and launches that used the XCD-striped one.  A launch made while its
+ * stream is being captured into a graph cannot carry that offset (a replayed node sees another one):
+ * up to 128 MiB it is sided all the same, its kernel reading the offset from a device word that a
+ * one-wave kernel, captured ahead of the first such launch of the capture, writes at every replay;
+ * beyond, it uses the striped map. */
 /* Measures which side `count` sample granules of the device memory [region, region + num_bytes)
  * lie on, for memory the pool did not hand out (for the pool's own, sideaware_side_of answers
  * from what was measured when the arena was acquired).  Sample i is the 8 KiB granule number
@@ -240,7 +242,8 @@ int sideaware_alloc_stats(unsigned long long* out, int capacity);
  * than its output is sided too, following its first input; 0, the default: such ops use the striped map,
  * which is as fast for them), "sided_agreement" (per cent of its length over which a second input as
  * wide as the followed one must have the same sides for the launch to be sided; default 70) and
- * "sided_align" (the followed array must start on a multiple of this many bytes; default 16).
+ * "sided_align" (the followed array must start on a multiple of this many bytes; default 16);
+ * "sided_from_memory" (1: direct launches read the dealing offset from memory as captured ones do, an A/B switch).
  * Returns 0 if the key is known and the value acceptable. */
 int sideaware_tune(const char* key, long long value);
 long long sideaware_tune_get(const char* key);

@@ -238,13 +238,13 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch, bo
         "-ffp-contract=off",
         // The compiler is kept from forming packed fp32 instructions out of scalar code.
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        // The first kernel arguments (the launch plan's scalars, then the i0 and o0 pointers: as
-        // many as fit in fourteen registers) are handed to every wave in registers at its start
+        // The first kernel arguments (the launch plan's scalars, then the i0 and o0 pointers and the
+        // feedback word's: as many as fit in fourteen registers) are handed to every wave in registers at its start
         // instead of being fetched by its first instructions.  With one workgroup per 4 KiB chunk
         // that fetch is on the critical path of every workgroup: 16 MiB copies run 8 % faster
         // with the preload, 64 MiB copies 3 %.  The code object keeps a prologue that fetches the
         // same arguments for firmware that does not preload.
-        "-mllvm", "-amdgpu-kernarg-preload-count=11",
+        "-mllvm", "-amdgpu-kernarg-preload-count=10",
         "-I" + rocm_root() + "/include",
         "-I" + cwd,                       // op headers may #include "file" relative to the cwd
         "-Wno-unused-parameter",

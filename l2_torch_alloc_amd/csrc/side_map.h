@@ -144,6 +144,9 @@ public:
     // sharing a word could write it while the other reads).  *capturing says which.
     unsigned int* capture_word(void* stream, bool* capturing);
     void init_capture_words();
+    // The last of those words, set (synchronously) to `dealing`: for the A/B switch that makes direct
+    // launches read their dealing offset from memory as captured ones do.
+    unsigned int* debug_word(unsigned int dealing);
     static constexpr int kCaptureWords = 4096;
 
     // Times loads from every XCD at `count` sample granules of [region, region + bytes) on

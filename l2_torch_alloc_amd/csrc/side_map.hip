@@ -202,6 +202,20 @@ void SideRegistry::init_capture_words() {
     capture_words_ = (unsigned int*)ptr;
 }
 
+unsigned int* SideRegistry::debug_word(unsigned int dealing) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (!capture_words_) return nullptr;
+    unsigned int* word = capture_words_ + (kCaptureWords - 1);
+    static unsigned int last = ~0u;
+    const unsigned int v = 0x80000000u | (dealing & 0xfu);
+    if (v != last) {
+        DeviceGuard dev(device_);
+        if (hipMemcpy(word, &v, sizeof v, hipMemcpyHostToDevice) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        last = v;
+    }
+    return word;
+}
+
 unsigned int* SideRegistry::capture_word(void* stream, bool* capturing) {
     *capturing = false;
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
@@ -219,7 +233,7 @@ unsigned int* SideRegistry::capture_word(void* stream, bool* capturing) {
     const auto key = std::make_pair(id, stream);
     auto it = capture_word_of_.find(key);
     if (it != capture_word_of_.end()) return capture_words_ + it->second;
-    if (capture_words_used_ >= kCaptureWords) return nullptr;
+    if (capture_words_used_ >= kCaptureWords - 1) return nullptr;      // the last word is the A/B switch's
     unsigned int* word = capture_words_ + capture_words_used_;
     DeviceGuard dev(device_);
     hipLaunchKernelGGL(sa_scout, dim3(1), dim3(64), 0, (hipStream_t)stream, word);      // captured, like the launch that follows

@@ -98,23 +98,25 @@ struct Tuning {
     long long sided_widening = 0;    // 1: ops whose every input is narrower than the output are sided too, following i0 (an A/B switch)
     long long sided_agreement = 70;  // per cent of an array over which another array of the same width must match its sides
     long long sided_align = 16;      // the followed array must start on a multiple of this many bytes (a power of two, at least 16)
+    long long sided_from_memory = 0; // 1: direct launches read their dealing offset from a device word as captured ones do (an A/B switch)
 };
 
 // The knobs themselves: written by sideaware_tune (and once from the environment), read by every
 // launch on any thread, hence atomics.  Kernels carry the generation they were compiled under;
 // a change of a compiled-in knob bumps it and the next launch builds a fresh instantiation.
-constexpr int kTuneKnobs = 16;
+constexpr int kTuneKnobs = 17;
 static const char* const kTuneNames[kTuneKnobs] = {"stripe_bytes", "slot_run", "one_shot", "cache_bytes",
                                                    "nt_store", "groups_cap", "wg_threads", "stripes_per_xcd",
                                                    "write_through", "sided", "sided_min_bytes", "sided_stripe",
-                                                   "sided_wrong", "sided_widening", "sided_agreement", "sided_align"};
+                                                   "sided_wrong", "sided_widening", "sided_agreement", "sided_align",
+                                                   "sided_from_memory"};
 static const char* const kTuneEnv[kTuneKnobs] = {"SIDEAWARE_STRIPE_BYTES", "SIDEAWARE_SLOT_RUN", "SIDEAWARE_ONE_SHOT",
                                                  "SIDEAWARE_CACHE_BYTES", "SIDEAWARE_NT_STORE", "SIDEAWARE_GROUPS_CAP",
                                                  "SIDEAWARE_WG_THREADS", "SIDEAWARE_STRIPES_PER_XCD",
                                                  "SIDEAWARE_WRITE_THROUGH", "SIDEAWARE_SIDED", "SIDEAWARE_SIDED_MIN_BYTES",
                                                  "SIDEAWARE_SIDED_STRIPE", "SIDEAWARE_SIDED_WRONG", "SIDEAWARE_SIDED_WIDENING",
-                                                 "SIDEAWARE_SIDED_AGREEMENT", "SIDEAWARE_SIDED_ALIGN"};
-static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}, {0}, {70}, {16}};
+                                                 "SIDEAWARE_SIDED_AGREEMENT", "SIDEAWARE_SIDED_ALIGN", "SIDEAWARE_SIDED_FROM_MEMORY"};
+static std::atomic<long long> g_tune[kTuneKnobs] = {{0}, {1}, {1}, {256ll << 20}, {2}, {8}, {256}, {8}, {1}, {1}, {8ll << 20}, {-1}, {0}, {0}, {70}, {16}, {0}};
 static std::atomic<unsigned> g_tune_generation{0};
 static std::mutex g_tune_mu;
 
@@ -148,6 +150,7 @@ static Tuning tuning_snapshot() {
     t.sided_widening = g_tune[13].load(std::memory_order_relaxed);
     t.sided_agreement = g_tune[14].load(std::memory_order_relaxed);
     t.sided_align = g_tune[15].load(std::memory_order_relaxed);
+    t.sided_from_memory = g_tune[16].load(std::memory_order_relaxed);
     return t;
 }
 
@@ -669,12 +672,12 @@ struct SegmentArgs {
 struct BatchArgs {                        // the batched entry point's arguments, in their order
     unsigned int count;
     unsigned int blocks_end[kMaxSegments];
-    unsigned int reserved;
-    SegmentArgs seg[kMaxSegments];
+    unsigned int padding;                // keeps the pointer 8-byte aligned
     unsigned int* feedback;
+    SegmentArgs seg[kMaxSegments];
 };
 static_assert(sizeof(SegmentArgs) == 128 && sizeof(BatchArgs) == 128 * kMaxSegments + 8 + 4 * kMaxSegments + 8 &&
-              offsetof(BatchArgs, seg) == 40 && kMaxSegments == 8,
+              offsetof(BatchArgs, feedback) == 40 && offsetof(BatchArgs, seg) == 48 && kMaxSegments == 8,
               "the device side declares the same layout");
 
 // The instantiation a launch over these arrays needs.  Index width: 32-bit below 2 GiB, 64-bit from
@@ -725,6 +728,8 @@ static long long slots_wanted_for(const DeviceContext* ctx, const CompiledKernel
 // is switched on, the array is long enough to matter, the op is not known to be one that cannot be
 // sided (see sa_sided_possible in the kernel template), and one of the two arrays a sided launch may
 // follow lies in an arena whose sides were measured (and starts on a multiple of the `sided_align` knob).
+constexpr size_t kCapturedSidedMaxBytes = 128ull << 20;
+
 static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const void* out0, const void* in0,
                             size_t num_bytes, const Tuning& t, sideaware_stream_t stream, unsigned int** capture_word) {
     *capture_word = nullptr;
@@ -748,9 +753,26 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
     // plan is frozen into the node, so a captured launch's kernel reads the offset from a device word
     // that a one-wave kernel captured ahead of it writes at every replay; when there is no such word
     // to be had the launch uses the map that does not depend on the offset.
+    // Reading the word costs every workgroup some 200 cycles before it can find its tile (direct
+    // launches forced to do the same, `sided_from_memory`: a 256 MiB copy 80.1 instead of 77.2 us, a
+    // 64 MiB one 22.3 instead of 20.6), which is what the sided map gains over the striped one when
+    // the arrays come from HBM, and a small part of what it gains when they come from the Infinity
+    // Cache (chains in which each launch reads what the launch before it wrote, replayed from a graph:
+    // 14.3 against 19.0 us at 64 MiB, 27.5 against 36.8 at 128 MiB, 74.5 against 74.1 at 256 MiB).  So
+    // captured launches are sided up to kCapturedSidedMaxBytes, which is where a graph's arrays are
+    // each other's inputs more often than not, and striped beyond.
     bool capturing = false;
-    *capture_word = sides.capture_word(stream, &capturing);
-    if (capturing) return *capture_word != nullptr;
+    if (num_bytes > kCapturedSidedMaxBytes) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &status) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        if (status != hipStreamCaptureStatusNone) return false;
+    } else {
+        *capture_word = sides.capture_word(stream, &capturing);
+        if (capturing) return *capture_word != nullptr;
+    }
     return sides.stream_is_steady(stream);
 }
 
@@ -986,6 +1008,12 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
             side.dealing_from_memory = true;
         } else {
             feedback = ctx->backing->sides().feedback_slot(stream, &side.dealing);
+            if (t.sided_from_memory) {
+                if (unsigned int* word = ctx->backing->sides().debug_word(side.dealing)) {
+                    feedback = word;
+                    side.dealing_from_memory = true;
+                }
+            }
         }
         plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? out0 : in0), num_vectors, k->tile_vectors,
                                  ctx->num_xcds, sided_stripe_for(num_bytes, out0 == in0, t), t.slot_run, slots_wanted, side,
@@ -997,30 +1025,33 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     }
 
     // The kernel's arguments, laid out as the device code declares them (natural alignment, in
-    // order: the plan's scalars, the workgroup count, then i0, o0 and the other pointers) and
+    // order: the plan's scalars, the workgroup count, i0, o0 and the feedback word, then what is
+    // needed late: the owner of the last tile, the sideband value, the other pointers) and
     // handed to the runtime as one block.
-    struct Args32 { int nv, ft, b0, uc, run; unsigned int r; int tail; int val; unsigned int blocks; void* p[10]; };
-    struct Args64 { long long nv, ft, b0, uc, run; unsigned int r; int tail; int val; unsigned int blocks; void* p[10]; };
-    static_assert(offsetof(Args32, p) == 40 && sizeof(Args32) == 120 && offsetof(Args64, p) == 56 && sizeof(Args64) == 136,
+    struct Args32 { int nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; int pad; void* first[3]; int tail; int val; void* rest[7]; };
+    struct Args64 { long long nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; void* first[3]; int tail; int val; void* rest[7]; };
+    static_assert(offsetof(Args32, first) == 32 && offsetof(Args32, tail) == 56 && offsetof(Args32, rest) == 64 && sizeof(Args32) == 120 &&
+                  offsetof(Args64, first) == 48 && offsetof(Args64, tail) == 72 && offsetof(Args64, rest) == 80 && sizeof(Args64) == 136,
                   "kernel argument layout");
     union { Args32 a32; Args64 a64; } args;
     size_t args_bytes;
-    void* const ptrs[10] = {(void*)in0, out0, out1, out2, out3, (void*)in1, (void*)in2, (void*)in3, sideband_memory,
-                            feedback};
+    void* const first[3] = {(void*)in0, out0, feedback};
+    void* const rest[7] = {out1, out2, out3, (void*)in1, (void*)in2, (void*)in3, sideband_memory};
     if (wide) {
         Args64& a = args.a64;
         a.nv = num_vectors;
         a.ft = plan.full_tiles; a.b0 = plan.b0; a.uc = plan.u_count; a.run = plan.run;
-        a.r = plan.r_word; a.tail = plan.tail_block; a.val = sideband_value; a.blocks = plan.grid;
-        std::memcpy(a.p, ptrs, sizeof ptrs);
+        a.r = plan.r_word; a.blocks = plan.grid; a.tail = plan.tail_block; a.val = sideband_value;
+        std::memcpy(a.first, first, sizeof first);
+        std::memcpy(a.rest, rest, sizeof rest);
         args_bytes = sizeof(Args64);
     } else {
         Args32& a = args.a32;
         a.nv = (int)num_vectors;
         a.ft = (int)plan.full_tiles; a.b0 = (int)plan.b0; a.uc = (int)plan.u_count; a.run = (int)plan.run;
-        a.r = plan.r_word; a.tail = plan.tail_block; a.val = sideband_value; a.blocks = plan.grid;
-        std::memset((char*)&a + 36, 0, 4);                       // the padding in front of the pointers
-        std::memcpy(a.p, ptrs, sizeof ptrs);
+        a.r = plan.r_word; a.blocks = plan.grid; a.pad = 0; a.tail = plan.tail_block; a.val = sideband_value;
+        std::memcpy(a.first, first, sizeof first);
+        std::memcpy(a.rest, rest, sizeof rest);
         args_bytes = sizeof(Args32);
     }
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &args_bytes, HIP_LAUNCH_PARAM_END};

@@ -87,8 +87,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
                 blockIdx = {b, 0, 0};
                 threadIdx = {t, 0, 0};
                 const unsigned* e = batch.blocks_end;
-                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7], 0u, batch.segments,
-                                               g_dealing_from_memory ? &g_dealing_word : nullptr);
+                SA_CONCAT(KERNEL_NAME, _batch)(batch.count, e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7],
+                                               g_dealing_from_memory ? &g_dealing_word : nullptr, batch.segments);
             }
         }
         return;
@@ -102,8 +102,8 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
             KERNEL_NAME(nv, (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
-                        p.r_word, p.tail_block, val, p.grid, i0, o0, o1, o2, o3, i1, i2, i3, mem,
-                        g_dealing_from_memory ? &g_dealing_word : nullptr);
+                        p.r_word, p.grid, i0, o0, g_dealing_from_memory ? &g_dealing_word : nullptr, p.tail_block, val,
+                        o1, o2, o3, i1, i2, i3, mem);
         }
     }
 }
