@@ -244,7 +244,7 @@ CompileResult compile_for_gfx950(const std::string& source, const char* arch, bo
         // that fetch is on the critical path of every workgroup: 16 MiB copies run 8 % faster
         // with the preload, 64 MiB copies 3 %.  The code object keeps a prologue that fetches the
         // same arguments for firmware that does not preload.
-        "-mllvm", "-amdgpu-kernarg-preload-count=10",
+        "-mllvm", "-amdgpu-kernarg-preload-count=11",
         "-I" + rocm_root() + "/include",
         "-I" + cwd,                       // op headers may #include "file" relative to the cwd
         "-Wno-unused-parameter",

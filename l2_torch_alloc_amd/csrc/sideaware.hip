@@ -1025,13 +1025,13 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
     }
 
     // The kernel's arguments, laid out as the device code declares them (natural alignment, in
-    // order: the plan's scalars, the workgroup count, i0, o0 and the feedback word, then what is
-    // needed late: the owner of the last tile, the sideband value, the other pointers) and
+    // order: the plan's scalars, the workgroup count, the sideband value, i0, o0 and the feedback
+    // word, then what is needed late: the owner of the last tile, the other pointers) and
     // handed to the runtime as one block.
-    struct Args32 { int nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; int pad; void* first[3]; int tail; int val; void* rest[7]; };
-    struct Args64 { long long nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; void* first[3]; int tail; int val; void* rest[7]; };
+    struct Args32 { int nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; int val; void* first[3]; int tail; int pad; void* rest[7]; };
+    struct Args64 { long long nv, ft, b0, uc, run; unsigned int r; unsigned int blocks; int val; int pad0; void* first[3]; int tail; int pad; void* rest[7]; };
     static_assert(offsetof(Args32, first) == 32 && offsetof(Args32, tail) == 56 && offsetof(Args32, rest) == 64 && sizeof(Args32) == 120 &&
-                  offsetof(Args64, first) == 48 && offsetof(Args64, tail) == 72 && offsetof(Args64, rest) == 80 && sizeof(Args64) == 136,
+                  offsetof(Args64, first) == 56 && offsetof(Args64, tail) == 80 && offsetof(Args64, rest) == 88 && sizeof(Args64) == 144,
                   "kernel argument layout");
     union { Args32 a32; Args64 a64; } args;
     size_t args_bytes;
@@ -1041,7 +1041,7 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         Args64& a = args.a64;
         a.nv = num_vectors;
         a.ft = plan.full_tiles; a.b0 = plan.b0; a.uc = plan.u_count; a.run = plan.run;
-        a.r = plan.r_word; a.blocks = plan.grid; a.tail = plan.tail_block; a.val = sideband_value;
+        a.r = plan.r_word; a.blocks = plan.grid; a.val = sideband_value; a.pad0 = 0; a.tail = plan.tail_block; a.pad = 0;
         std::memcpy(a.first, first, sizeof first);
         std::memcpy(a.rest, rest, sizeof rest);
         args_bytes = sizeof(Args64);
@@ -1049,7 +1049,7 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
         Args32& a = args.a32;
         a.nv = (int)num_vectors;
         a.ft = (int)plan.full_tiles; a.b0 = (int)plan.b0; a.uc = (int)plan.u_count; a.run = (int)plan.run;
-        a.r = plan.r_word; a.blocks = plan.grid; a.pad = 0; a.tail = plan.tail_block; a.val = sideband_value;
+        a.r = plan.r_word; a.blocks = plan.grid; a.val = sideband_value; a.tail = plan.tail_block; a.pad = 0;
         std::memcpy(a.first, first, sizeof first);
         std::memcpy(a.rest, rest, sizeof rest);
         args_bytes = sizeof(Args32);

@@ -102,7 +102,7 @@ static void run_grid(unsigned grid, size_type nv, vo0* o0, vo1* o1, vo2* o2, vo3
             blockIdx = {b, 0, 0};
             threadIdx = {t, 0, 0};
             KERNEL_NAME(nv, (size_type)p.full_tiles, (size_type)p.b0, (size_type)p.u_count, (size_type)p.run,
-                        p.r_word, p.grid, i0, o0, g_dealing_from_memory ? &g_dealing_word : nullptr, p.tail_block, val,
+                        p.r_word, p.grid, val, i0, o0, g_dealing_from_memory ? &g_dealing_word : nullptr, p.tail_block,
                         o1, o2, o3, i1, i2, i3, mem);
         }
     }
