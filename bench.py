@@ -324,11 +324,31 @@ def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
                     times[sided].append(time_region(launch, n_steps, 9))
         finally:
             lib.sideaware_tune(b"sided", 1)
+        # the same chain captured into a HIP graph (60 launches) and replayed on the default stream:
+        # a captured launch cannot know the XCD its workgroups will be dealt from, so its kernel reads
+        # that from a word a one-wave kernel at the head of the graph writes (up to 128 MiB; striped beyond)
+        replayed = {}
+        try:
+            for sided in (1, 0):
+                lib.sideaware_tune(b"sided", sided)
+                graph = torch.cuda.CUDAGraph()
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    with torch.cuda.graph(graph, stream=side):
+                        for i in range(60):
+                            lib.sideaware_memcpy(bufs[(i + 1) % 3].data_ptr(), bufs[i % 3].data_ptr(), nbytes, 0, side.cuda_stream)
+                torch.cuda.current_stream().wait_stream(side)
+                replayed[sided] = statistics.median([time_region(graph.replay, 4, 1) / 60 for _ in range(rounds)])
+                del graph
+        finally:
+            lib.sideaware_tune(b"sided", 1)
         ok = all(bool(torch.equal(b, first)) for b in bufs)
         entry = {"bytes": nbytes, "bit_exact": ok}
         for sided, name in ((1, "sided"), (0, "xcd_striped")):
             sec = statistics.median(times[sided])
-            entry[name] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes, sec)}
+            entry[name] = {"us": sec * 1e6, "GBps": gbps(2 * nbytes, sec),
+                           "replayed_from_a_hip_graph_us": replayed[sided] * 1e6}
         out["%dMiB" % (nbytes // MiB)] = entry
         del bufs
     return out
