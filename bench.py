@@ -326,7 +326,7 @@ def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
             lib.sideaware_tune(b"sided", 1)
         # the same chain captured into a HIP graph (60 launches) and replayed on the default stream:
         # a captured launch cannot know the XCD its workgroups will be dealt from, so its kernel reads
-        # that from a word a one-wave kernel at the head of the graph writes (up to 128 MiB; striped beyond)
+        # that from a word a one-wave kernel at the head of the graph writes
         replayed = {}
         try:
             for sided in (1, 0):

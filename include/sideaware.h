@@ -159,9 +159,9 @@ int sideaware_xcd_dealing_verified(void);
  * ran on (0 before any): sided launches plan with it.  sideaware_launch_counts: launches so far
  * that used the sided map, and launches that used the XCD-striped one.  A launch made while its
  * stream is being captured into a graph cannot carry that offset (a replayed node sees another one):
- * up to 128 MiB it is sided all the same, its kernel reading the offset from a device word that a
- * one-wave kernel, captured ahead of the first such launch of the capture, writes at every replay;
- * beyond, it uses the striped map. */
+ * it is sided all the same, its kernel reading the offset from a device word that a one-wave kernel,
+ * captured ahead of the first such launch of the capture, writes at every replay (4,095 such words
+ * per process; captures beyond that use the striped map). */
 /* Measures which side `count` sample granules of the device memory [region, region + num_bytes)
  * lie on, for memory the pool did not hand out (for the pool's own, sideaware_side_of answers
  * from what was measured when the arena was acquired).  Sample i is the 8 KiB granule number

@@ -728,8 +728,6 @@ static long long slots_wanted_for(const DeviceContext* ctx, const CompiledKernel
 // is switched on, the array is long enough to matter, the op is not known to be one that cannot be
 // sided (see sa_sided_possible in the kernel template), and one of the two arrays a sided launch may
 // follow lies in an arena whose sides were measured (and starts on a multiple of the `sided_align` knob).
-constexpr size_t kCapturedSidedMaxBytes = 128ull << 20;
-
 static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const void* out0, const void* in0,
                             size_t num_bytes, const Tuning& t, sideaware_stream_t stream, unsigned int** capture_word) {
     *capture_word = nullptr;
@@ -753,26 +751,12 @@ static bool sided_candidate(DeviceContext* ctx, const KernelEntry* entry, const 
     // plan is frozen into the node, so a captured launch's kernel reads the offset from a device word
     // that a one-wave kernel captured ahead of it writes at every replay; when there is no such word
     // to be had the launch uses the map that does not depend on the offset.
-    // Reading the word costs every workgroup some 200 cycles before it can find its tile (direct
-    // launches forced to do the same, `sided_from_memory`: a 256 MiB copy 80.1 instead of 77.2 us, a
-    // 64 MiB one 22.3 instead of 20.6), which is what the sided map gains over the striped one when
-    // the arrays come from HBM, and a small part of what it gains when they come from the Infinity
-    // Cache (chains in which each launch reads what the launch before it wrote, replayed from a graph:
-    // 14.3 against 19.0 us at 64 MiB, 27.5 against 36.8 at 128 MiB, 74.5 against 74.1 at 256 MiB).  So
-    // captured launches are sided up to kCapturedSidedMaxBytes, which is where a graph's arrays are
-    // each other's inputs more often than not, and striped beyond.
+    // Reading the word is one scalar load per wave, answered by the scalar cache: direct launches
+    // forced to do the same (`sided_from_memory`) run as fast as with the offset in their launch word
+    // (256 MiB copy 77.85 against 77.78 us; through the vector path it was 80.1).
     bool capturing = false;
-    if (num_bytes > kCapturedSidedMaxBytes) {
-        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing((hipStream_t)stream, &status) != hipSuccess) {
-            (void)hipGetLastError();
-            return false;
-        }
-        if (status != hipStreamCaptureStatusNone) return false;
-    } else {
-        *capture_word = sides.capture_word(stream, &capturing);
-        if (capturing) return *capture_word != nullptr;
-    }
+    *capture_word = sides.capture_word(stream, &capturing);
+    if (capturing) return *capture_word != nullptr;
     return sides.stream_is_steady(stream);
 }
 
