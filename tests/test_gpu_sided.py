@@ -361,6 +361,40 @@ def test_sided_launches_replay_from_a_hip_graph(sa, lib):
     assert not sa.sideaware_last_error()
 
 
+def test_a_sided_batch_replays_from_a_hip_graph(sa, lib):
+    """q and k of a grouped-query model rotated in one batched launch (both long enough to be
+    sided), captured into a graph: the replays give what the direct launch gives, bit for bit."""
+    from l2_torch_alloc_amd import ops
+    T, D = 4096, 128
+    freqs = ops.freqs_cis_table(D, T, 500000.0).cuda()
+    g = torch.Generator().manual_seed(5)
+    q0 = torch.randn(1, T, 32, D, generator=g).to(torch.bfloat16).cuda()      # 32 MiB
+    k0 = torch.randn(1, T, 8, D, generator=g).to(torch.bfloat16).cuda()       # 8 MiB
+    want_q, want_k = q0.clone(), k0.clone()
+    before = counts(lib)
+    ops.rope_forward_heads_many([want_q, want_k], freqs)                       # direct, and compiles outside the capture
+    torch.cuda.synchronize()
+    assert counts(lib) == (before[0] + 1, before[1])
+    q, k = q0.clone(), k0.clone()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    before = counts(lib)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.rope_forward_heads_many([q, k], freqs)
+    torch.cuda.current_stream().wait_stream(side)
+    assert counts(lib) == (before[0] + 1, before[1])
+    for trial in range(3):
+        q.copy_(q0)
+        k.copy_(k0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(q, want_q) and torch.equal(k, want_k), trial
+    assert not sa.sideaware_last_error()
+
+
 def test_the_dealing_offset_survives_other_kernels_on_the_stream(sa, lib):
     """The sided map plans with the XCD that workgroup 0 of the stream's last sided launch ran on.
     That offset belongs to the queue, not to its history: kernels of other shapes in between (PyTorch's
