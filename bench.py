@@ -298,22 +298,37 @@ def bench_one_direction(nbytes=GiB, sets=4, steps=12, rounds=3):
     return out
 
 
-def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
+def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3, named_kernels=False):
     """Producer -> consumer chains: three buffers, every launch copies the one the launch before it
     wrote into the next, so each launch reads what was just written (from the Infinity Cache while
     three buffers fit it, partly from HBM at 256 MiB).  Sided and XCD-striped in turn (medians)."""
     import torch
     lib, stream = _abi()
     out = {}
+    kids = {}
+    if named_kernels:                            # for a kernel trace: one kernel name per size and map
+        from l2_torch_alloc_amd import headers, wrapper
+        for nbytes in sizes:
+            for sided in (1, 0):
+                name = "sideaware_copy_chain_%dMiB_%s" % (nbytes // MiB, "sided" if sided else "xcd_striped")
+                kids[(nbytes, sided)] = wrapper.sideaware_create_kernel(
+                    headers.memcpy_header().decode().replace("sideaware_copy_spelled_out", name).encode())
+    current = [1]
     for nbytes in sizes:
         bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(3)]
         first = bufs[0].clone()
         counter = [0]
 
+        def copy(dst, src, on_stream):
+            if named_kernels:
+                lib.sideaware_one_to_one(kids[(nbytes, current[0])], nbytes, dst, src, 0, on_stream)
+            else:
+                lib.sideaware_memcpy(dst, src, nbytes, 0, on_stream)
+
         def launch():
             i = counter[0] % 3
             counter[0] += 1
-            lib.sideaware_memcpy(bufs[(i + 1) % 3].data_ptr(), bufs[i].data_ptr(), nbytes, 0, stream)
+            copy(bufs[(i + 1) % 3].data_ptr(), bufs[i].data_ptr(), stream)
 
         times = {1: [], 0: []}
         n_steps = max(30, steps * (16 * MiB) // nbytes)
@@ -321,6 +336,7 @@ def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
             for _ in range(rounds):
                 for sided in (1, 0):
                     lib.sideaware_tune(b"sided", sided)
+                    current[0] = sided
                     times[sided].append(time_region(launch, n_steps, 9))
         finally:
             lib.sideaware_tune(b"sided", 1)
@@ -331,13 +347,14 @@ def bench_chains(sizes=(16 * MiB, 64 * MiB, 256 * MiB), steps=300, rounds=3):
         try:
             for sided in (1, 0):
                 lib.sideaware_tune(b"sided", sided)
+                current[0] = sided
                 graph = torch.cuda.CUDAGraph()
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
                     with torch.cuda.graph(graph, stream=side):
                         for i in range(60):
-                            lib.sideaware_memcpy(bufs[(i + 1) % 3].data_ptr(), bufs[i % 3].data_ptr(), nbytes, 0, side.cuda_stream)
+                            copy(bufs[(i + 1) % 3].data_ptr(), bufs[i % 3].data_ptr(), side.cuda_stream)
                 torch.cuda.current_stream().wait_stream(side)
                 replayed[sided] = statistics.median([time_region(graph.replay, 4, 1) / 60 for _ in range(rounds)])
                 del graph
@@ -908,6 +925,9 @@ def main():
     ap.add_argument("--side-ab", action="store_true",
                     help="only the 256 MiB copy under the three ownership maps (sided, XCD-striped, sided the wrong "
                          "way round), each under a kernel name of its own (for a kernel trace)")
+    ap.add_argument("--chains", action="store_true",
+                    help="only the producer -> consumer chains, sided and striped, directly and replayed from a HIP graph, "
+                         "each under a kernel name of its own (for a kernel trace)")
     ap.add_argument("--one-direction", action="store_true",
                     help="only the 1 GiB scan (loads only) and fill (stores only) under the sided and the striped map")
     ap.add_argument("--only", action="append", default=None,
@@ -940,6 +960,9 @@ def main():
         import bench_experiments as experiments      # the sweep modes: not needed by the default run
     if args.side_ab:
         print(json.dumps({"copy_256MiB_ownership_map_ab": bench_side_ab(named_kernels=True)}))
+        return
+    if args.chains:
+        print(json.dumps({"chain_each_launch_reads_what_the_last_wrote": bench_chains(named_kernels=True)}))
         return
     if args.one_direction:
         print(json.dumps({"one_direction_1GiB": bench_one_direction()}))
