@@ -1018,8 +1018,8 @@ def main():
         # 1 GiB that one is served partly from the Infinity Cache: a cache figure, not an HBM one).
         sweep = {}
         for label, nbytes, pairs, steps in (("4MiB", 4 * MiB, 128, 512), ("64MiB", 64 * MiB, 8, 96),
-                                            ("256MiB", 256 * MiB, 8, 48), ("1GiB", GiB, 4, 20), ("8GiB", 8 * GiB, 2, 6)):
-            cycling = bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=3, prewarm=pairs, dtype="fp32")
+                                            ("256MiB", 256 * MiB, 8, 48), ("1GiB", GiB, 4, 40), ("8GiB", 8 * GiB, 2, 16)):
+            cycling = bench_copy_rotating(nbytes, pairs, steps, warmup=2, seed=3, prewarm=max(pairs, 8), dtype="fp32")
             one_pair = bench_copy(nbytes, steps, 3, "fp32", seed=3)
             sweep[label] = {"hbm_cycling_pairs": cycling, "one_pair_in_a_loop": one_pair,
                             "working_set_bytes_cycling": 2 * nbytes * pairs}
