@@ -95,6 +95,7 @@ struct SideMap {
     unsigned int flip = 0;         // 0 or 1: the arena's constant
     unsigned int dealing = 0;      // workgroup w of a launch runs on XCD (w + dealing) % num_xcds
     bool dealing_from_memory = false;   // the kernel reads the dealing offset from a device word instead (captured launches)
+    bool report = false;                // workgroup 0 writes the XCD it runs on to the launch's feedback word
 };
 
 inline unsigned int parity32(unsigned int v) { return (unsigned int)__builtin_popcount(v) & 1u; }
@@ -144,7 +145,8 @@ inline LaunchPlan plan_launch_sided(uint64_t base_address, long long num_vectors
     // a launch that reads the offset at run time is planned as if it were 0: only the choice of the
     // workgroup that takes the partial last tile depends on it, and any choice is correct
     const unsigned int dealing = side.dealing_from_memory ? 0u : side.dealing % (unsigned int)num_xcds;
-    p.r_word = p.r | (dealing << 8) | ((side.flip & 1u) << 12) | (side.dealing_from_memory ? 0x8000u : 0u) | (origin << 16);
+    p.r_word = p.r | (dealing << 8) | ((side.flip & 1u) << 12) | (side.dealing_from_memory ? 0x8000u : 0u) | (origin << 16) |
+               (side.report && !side.dealing_from_memory ? 0x80000000u : 0u);
 
     if (p.full_tiles * tile_vectors < num_vectors) {
         const long long a = p.b0 + p.full_tiles;

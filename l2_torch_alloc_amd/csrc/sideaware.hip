@@ -1001,6 +1001,7 @@ void sideaware_elementwise(int kernel_id, size_t num_bytes,
             side.dealing_from_memory = true;
         } else {
             feedback = ctx->backing->sides().feedback_slot(stream, &side.dealing);
+            side.report = feedback != nullptr;
             if (t.sided_from_memory) {
                 if (unsigned int* word = ctx->backing->sides().debug_word(side.dealing)) {
                     feedback = word;
@@ -1133,6 +1134,7 @@ void sideaware_elementwise_batch(int kernel_id, int num_segments, const sideawar
             if (k->sided) {
                 sides[i].dealing = dealing;
                 sides[i].dealing_from_memory = capture_word != nullptr;
+                sides[i].report = capture_word == nullptr && batch.feedback != nullptr;
                 plan = plan_launch_sided((uint64_t)(uintptr_t)(k->owner_is_o0 ? g.out[0] : g.in[0]), num_vectors,
                                          k->tile_vectors, ctx->num_xcds,
                                          sided_stripe_for(g.num_bytes, g.out[0] == g.in[0], t), t.slot_run, slots_wanted, sides[i],
